@@ -1,0 +1,479 @@
+// Operator entry points of the C ABI: argument checks (pure host, before any HIP
+// call), shape derivation, tile-table lookup, launch.  Mirrors the hand-written
+// operator layer of the reference (modules/flash/csrc/attn_fwd.cc:48-149,
+// attn_bwd.cc:55-160, attn_debug.cc:30-69, attn_check.cc:36-46); the generated
+// dispatch / kernel-image runtime underneath it is replaced by direct launches of
+// kernels linked into this library.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "aotriton_amd/flash.h"
+#include "fa_args.h"
+#include "fa_intervals.h"
+#include "fa_kernels.h"
+
+namespace {
+
+// AOTRITON_DEBUG_LEVEL=0..5 -> stderr (include/aotriton/_internal/log.h:56-65)
+int log_level() {
+  static int level = [] {
+    const char* e = std::getenv("AOTRITON_DEBUG_LEVEL");
+    return e ? std::atoi(e) : 0;
+  }();
+  return level;
+}
+#define FA_LOG(lvl, ...)                                  \
+  do {                                                    \
+    if (log_level() >= (lvl)) {                           \
+      std::fprintf(stderr, "[aotriton_amd] " __VA_ARGS__); \
+      std::fputc('\n', stderr);                           \
+    }                                                     \
+  } while (0)
+
+constexpr int kMaxDevices = 64;
+struct DeviceInfo {
+  std::atomic<int> state{0};   // 0 unknown, 1 filled
+  bool is_gfx950 = false;
+  int num_cu = 0;
+  char arch[32] = {0};
+};
+DeviceInfo g_devices[kMaxDevices];
+std::mutex g_device_mutex;
+
+// v3src/util.cc:65-113: arch name up to ':' and CU count, memoised per device.
+const DeviceInfo* device_of_stream(hipStream_t stream) {
+  int dev = 0;
+  hipError_t e = hipErrorUnknown;
+  if (stream != nullptr) e = hipStreamGetDevice(stream, &dev);
+  if (e != hipSuccess) e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  DeviceInfo& d = g_devices[dev];
+  if (d.state.load(std::memory_order_acquire) == 1) return &d;
+  std::lock_guard<std::mutex> lock(g_device_mutex);
+  if (d.state.load(std::memory_order_relaxed) == 1) return &d;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return nullptr;
+  size_t n = 0;
+  while (prop.gcnArchName[n] && prop.gcnArchName[n] != ':' && n + 1 < sizeof(d.arch)) {
+    d.arch[n] = prop.gcnArchName[n];
+    ++n;
+  }
+  d.arch[n] = 0;
+  d.is_gfx950 = std::strcmp(d.arch, "gfx950") == 0;
+  d.num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 40;
+  d.state.store(1, std::memory_order_release);
+  return &d;
+}
+
+bool is_16bit(int dt) { return dt == FA_DTYPE_FLOAT16 || dt == FA_DTYPE_BFLOAT16; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// rank-4 activation tensor: non-null, unit last stride, 16-byte aligned rows
+int check_act(const fa_tensor4& t, int dtype) {
+  if (t.ptr == nullptr) return FA_ERROR_INVALID_VALUE;
+  if (t.dtype != dtype) return FA_ERROR_INVALID_VALUE;
+  if (t.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
+  if (!aligned16(t.ptr)) return FA_ERROR_NOT_SUPPORTED;
+  for (int i = 0; i < 3; ++i)
+    if (t.sizes[i] > 1 && (t.strides[i] % 8) != 0) return FA_ERROR_NOT_SUPPORTED;
+  return FA_SUCCESS;
+}
+
+fa::Strides3 strides3(const fa_tensor4& t) {
+  return fa::Strides3{(int64_t)t.strides[0], (int64_t)t.strides[1], (int64_t)t.strides[2]};
+}
+
+struct Shape {
+  int batch, hq, hk, d, max_sq, max_sk, num_seqlens;  // num_seqlens signed as in attn_fwd.cc:99
+  bool windowed, bias, dropout;
+};
+
+// Shared by forward and backward: everything that only depends on
+// Q/K/V/B, the varlen descriptors and the scalar options.
+int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, const fa_tensor4& B,
+                 const fa_tensor1& cu_q, const fa_tensor1& cu_k, const fa_tensor1& ss_q,
+                 const fa_tensor1& ss_k, int32_t max_sq, int32_t max_sk, int varlen_type,
+                 int causal_type, float dropout_p, const fa_tensor0& seed, Shape* out) {
+  const int dtype = Q.dtype;
+  if (dtype != FA_DTYPE_FLOAT16 && dtype != FA_DTYPE_BFLOAT16 && dtype != FA_DTYPE_FLOAT32)
+    return FA_ERROR_INVALID_VALUE;
+  if (!is_16bit(dtype)) return FA_ERROR_NOT_SUPPORTED;   // fp32 kernels are not built
+  int e;
+  if ((e = check_act(Q, dtype)) != FA_SUCCESS) return e;
+  if ((e = check_act(K, dtype)) != FA_SUCCESS) return e;
+  if ((e = check_act(V, dtype)) != FA_SUCCESS) return e;
+  Shape s{};
+  s.batch = (int)Q.sizes[0];
+  s.hq = (int)Q.sizes[1];
+  s.hk = (int)K.sizes[1];
+  const int dqk = (int)Q.sizes[3], dv = (int)V.sizes[3];
+  if ((int)K.sizes[3] != dqk) return FA_ERROR_INVALID_VALUE;
+  if (s.hk <= 0 || s.hq <= 0 || s.hq % s.hk != 0 || (int)V.sizes[1] != s.hk) return FA_ERROR_INVALID_VALUE;
+  if (K.sizes[0] != Q.sizes[0] || V.sizes[0] != Q.sizes[0]) return FA_ERROR_INVALID_VALUE;
+  if (K.sizes[2] != V.sizes[2]) return FA_ERROR_INVALID_VALUE;
+  // compiled head dims; padded / mixed head dims are not built (attn_fwd.cc:76-82)
+  if (dqk != dv || !(dqk == 64 || dqk == 128 || dqk == 256)) return FA_ERROR_NOT_SUPPORTED;
+  s.d = dqk;
+  s.max_sq = (int)Q.sizes[2];
+  s.max_sk = (int)K.sizes[2];
+  s.num_seqlens = 0;
+  if (varlen_type < FA_VARLEN_NONE || varlen_type > FA_VARLEN_STRIDED) return FA_ERROR_INVALID_VALUE;
+  if (cu_q.ptr != nullptr) {
+    if (cu_k.ptr == nullptr || varlen_type == FA_VARLEN_NONE) return FA_ERROR_INVALID_VALUE;
+    if (cu_q.dtype != FA_DTYPE_INT32 || cu_k.dtype != FA_DTYPE_INT32) return FA_ERROR_INVALID_VALUE;
+    if (cu_q.sizes[0] < 2 || cu_k.sizes[0] != cu_q.sizes[0]) return FA_ERROR_INVALID_VALUE;
+    if (max_sq <= 0 || max_sk <= 0) return FA_ERROR_INVALID_VALUE;
+    const int n = (int)cu_q.sizes[0] - 1;
+    s.num_seqlens = varlen_type == FA_VARLEN_PADDED ? -n : n;
+    s.max_sq = max_sq;
+    s.max_sk = max_sk;
+    if (varlen_type == FA_VARLEN_STRIDED) {
+      if (ss_q.ptr == nullptr || ss_k.ptr == nullptr) return FA_ERROR_INVALID_VALUE;
+      if (ss_q.sizes[0] != cu_q.sizes[0] || ss_k.sizes[0] != cu_q.sizes[0]) return FA_ERROR_INVALID_VALUE;
+    }
+    if (varlen_type != FA_VARLEN_PADDED && s.batch != 1) return FA_ERROR_INVALID_VALUE;
+    if (varlen_type == FA_VARLEN_PADDED && s.batch != n) return FA_ERROR_INVALID_VALUE;
+  } else if (varlen_type != FA_VARLEN_NONE) {
+    return FA_ERROR_INVALID_VALUE;
+  }
+  if (causal_type != FA_CAUSAL_NONE && causal_type != FA_CAUSAL_WINDOWED) return FA_ERROR_NOT_SUPPORTED;
+  s.windowed = causal_type != FA_CAUSAL_NONE;
+  if (!(dropout_p >= 0.0f) || !(dropout_p < 1.0f)) return FA_ERROR_INVALID_VALUE;
+  s.dropout = dropout_p > 0.0f;   // attn_fwd.cc:110
+  if (s.dropout && seed.ptr == nullptr) return FA_ERROR_INVALID_VALUE;
+  s.bias = B.ptr != nullptr;      // attn_fwd.cc:122
+  if (s.bias) {
+    if (B.dtype != dtype) return FA_ERROR_INVALID_VALUE;
+    if (s.num_seqlens != 0) return FA_ERROR_NOT_SUPPORTED;   // bias has no packed layout
+    if ((int)B.sizes[0] != s.batch || (int)B.sizes[1] != s.hq || (int)B.sizes[2] != s.max_sq ||
+        (int)B.sizes[3] != s.max_sk)
+      return FA_ERROR_INVALID_VALUE;
+  }
+  *out = s;
+  return FA_SUCCESS;
+}
+
+fa::SeqArgs seq_args(const Shape& s, const fa_tensor1& cu_q, const fa_tensor1& cu_k,
+                     const fa_tensor1& ss_q, const fa_tensor1& ss_k, int varlen_type) {
+  fa::SeqArgs r{};
+  r.cu_q = static_cast<const int32_t*>(cu_q.ptr);
+  r.cu_k = static_cast<const int32_t*>(cu_k.ptr);
+  const bool strided = varlen_type == FA_VARLEN_STRIDED;
+  r.ss_q = strided ? static_cast<const int32_t*>(ss_q.ptr) : nullptr;
+  r.ss_k = strided ? static_cast<const int32_t*>(ss_k.ptr) : nullptr;
+  r.num_seqlens = s.num_seqlens;
+  r.max_seqlen_q = s.max_sq;
+  r.max_seqlen_k = s.max_sk;
+  return r;
+}
+
+int validate_fwd(const fa_fwd_params* p, int32_t version, const fa_options* opt, Shape* shape) {
+  if (p == nullptr) return FA_ERROR_INVALID_VALUE;
+  if (version != FA_FWD_PARAMS_VERSION) return FA_ERROR_INVALID_SYMBOL;   // attn_fwd.cc:53-55
+  Shape s{};
+  int e = check_common(p->Q, p->K, p->V, p->B, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q,
+                       p->seq_strides_k, p->Max_seqlen_q, p->Max_seqlen_k, p->varlen_type,
+                       p->causal_type, p->dropout_p, p->philox_seed_ptr, &s);
+  if (e != FA_SUCCESS) return e;
+  if ((e = check_act(p->Out, p->Q.dtype)) != FA_SUCCESS) return e;
+  for (int i = 0; i < 4; ++i)
+    if (p->Out.sizes[i] != (i == 3 ? p->V.sizes[3] : p->Q.sizes[i])) return FA_ERROR_INVALID_VALUE;
+  if (p->A.ptr != nullptr) return FA_ERROR_NOT_SUPPORTED;   // alibi: USE_ALIBI=false in attn_fwd.cc:123
+  if (p->L.ptr != nullptr && p->L.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  if (p->encoded_softmax.ptr != nullptr) {
+    const fa_tensor4& r = p->encoded_softmax;
+    if (r.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
+    if ((int)r.sizes[1] != s.hq || (int)r.sizes[2] != s.max_sq || (int)r.sizes[3] != s.max_sk)
+      return FA_ERROR_INVALID_VALUE;
+  }
+  // a forced backend that does not exist cannot take the input (template/op.cc:57-70)
+  if (opt != nullptr && opt->force_backend_index > 0) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
+  if (shape) *shape = s;
+  return FA_SUCCESS;
+}
+
+int bwd_backend(const fa_bwd_params* p, const fa_options* opt) {
+  if (opt != nullptr && opt->force_backend_index >= 0) return opt->force_backend_index;
+  if (opt != nullptr && opt->deterministic) return 0;   // attn_bwd.cc:147-148
+  // without a delta buffer only the fused backend can run
+  if (p->D.eager.ptr == nullptr && p->D.acquire == nullptr) return 1;
+  return 0;
+}
+
+int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt, Shape* shape,
+                 int* backend) {
+  if (p == nullptr) return FA_ERROR_INVALID_VALUE;
+  if (version != FA_BWD_PARAMS_VERSION) return FA_ERROR_INVALID_SYMBOL;   // attn_bwd.cc:60-62
+  Shape s{};
+  int e = check_common(p->Q, p->K, p->V, p->B, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q,
+                       p->seq_strides_k, p->Max_seqlen_q, p->Max_seqlen_k, p->varlen_type,
+                       p->causal_type, p->dropout_p, p->philox_seed_ptr, &s);
+  if (e != FA_SUCCESS) return e;
+  const int dt = p->Q.dtype;
+  if ((e = check_act(p->Out, dt)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DO, dt)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DQ, dt)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DK, dt)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DV, dt)) != FA_SUCCESS) return e;
+  for (int i = 0; i < 4; ++i) {
+    if (p->Out.sizes[i] != p->Q.sizes[i] || p->DO.sizes[i] != p->Q.sizes[i] ||
+        p->DQ.sizes[i] != p->Q.sizes[i] || p->DK.sizes[i] != p->K.sizes[i] ||
+        p->DV.sizes[i] != p->V.sizes[i])
+      return FA_ERROR_INVALID_VALUE;
+  }
+  if (p->L.ptr == nullptr || p->L.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  if (p->DB.ptr != nullptr) {
+    if (!s.bias) return FA_ERROR_INVALID_VALUE;
+    if (p->DB.dtype != dt) return FA_ERROR_INVALID_VALUE;
+    for (int i = 0; i < 4; ++i)
+      if (p->DB.sizes[i] != p->B.sizes[i]) return FA_ERROR_INVALID_VALUE;
+  }
+  const int be = bwd_backend(p, opt);
+  if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2
+  if (be == 0) {
+    if (p->D.eager.ptr == nullptr && p->D.acquire == nullptr) return FA_ERROR_INVALID_VALUE;
+    if (p->D.eager.ptr != nullptr && p->D.eager.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  }
+  if (shape) *shape = s;
+  if (backend) *backend = be;
+  return FA_SUCCESS;
+}
+
+hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
+  switch (d) {
+    case 64: return fa::run_fwd_d64(dtype, a, s.windowed, s.bias, s.dropout, stream);
+    case 128: return fa::run_fwd_d128(dtype, a, s.windowed, s.bias, s.dropout, stream);
+    case 256: return fa::run_fwd_d256(dtype, a, s.windowed, s.bias, s.dropout, stream);
+  }
+  return hipErrorNotSupported;
+}
+
+fa::DropoutArgs dropout_args(float p, const fa_tensor0& seed, const fa_tensor0& off1, uint64_t off2) {
+  fa::DropoutArgs d{};
+  d.p = p;
+  d.seed_ptr = static_cast<const uint64_t*>(seed.ptr);
+  d.offset1_ptr = static_cast<const uint64_t*>(off1.ptr);
+  d.offset2 = off2;
+  return d;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* fa_get_name_suffix(void) { return "_amd_gfx950"; }
+const char* fa_version(void) { return "0.1.0"; }
+
+int fa_get_arch(void* hip_stream, char* buf, int32_t buflen) {
+  const DeviceInfo* d = device_of_stream(static_cast<hipStream_t>(hip_stream));
+  if (d == nullptr || buf == nullptr || buflen <= 0) return FA_ERROR_INVALID_VALUE;
+  std::snprintf(buf, (size_t)buflen, "%s", d->arch);
+  return FA_SUCCESS;
+}
+
+int fa_get_multiprocessor_count(void* hip_stream) {
+  const DeviceInfo* d = device_of_stream(static_cast<hipStream_t>(hip_stream));
+  return d ? d->num_cu : 40;   // v3src/util.cc:95-112 falls back to 40
+}
+
+int fa_hip_get_last_error(void) { return (int)hipGetLastError(); }
+int fa_hip_device_synchronize(void) { return (int)hipDeviceSynchronize(); }
+
+int32_t fa_dropout_threshold(float dropout_p) { return fa::dropout_threshold(dropout_p); }
+
+int fa_tile_intervals(int32_t causal_type, int32_t window_left, int32_t window_right, int32_t start_m,
+                      int32_t seqlen_q, int32_t seqlen_k, int32_t block_m, int32_t block_n,
+                      int32_t out[6]) {
+  if (out == nullptr || block_m <= 0 || block_n <= 0) return FA_ERROR_INVALID_VALUE;
+  const bool windowed = causal_type != 0;
+  fa::Window w{0, 0};
+  if (windowed) w = fa::parse_window(causal_type, window_left, window_right, seqlen_q, seqlen_k);
+  const fa::BlockRanges r = fa::block_ranges(windowed, w.left, w.right, start_m, seqlen_q, seqlen_k,
+                                             block_m, block_n);
+  out[0] = r.lb_lo; out[1] = r.lb_hi; out[2] = r.fb_lo; out[3] = r.fb_hi; out[4] = r.rb_lo; out[5] = r.rb_hi;
+  return FA_SUCCESS;
+}
+
+int fa_check_gpu(void* hip_stream) {
+  const DeviceInfo* d = device_of_stream(static_cast<hipStream_t>(hip_stream));
+  if (d == nullptr || !d->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+  return FA_SUCCESS;
+}
+
+int fa_validate_fwd(const fa_fwd_params* params, int32_t params_version, const fa_options* options) {
+  return validate_fwd(params, params_version, options, nullptr);
+}
+
+int fa_validate_bwd(const fa_bwd_params* params, int32_t params_version, const fa_options* options) {
+  return validate_bwd(params, params_version, options, nullptr, nullptr);
+}
+
+int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_config* out) {
+  (void)num_cu;
+  if (out == nullptr) return FA_ERROR_INVALID_VALUE;
+  Shape s{};
+  int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
+  if (e != FA_SUCCESS) return e;
+  const fa::TileShape t = fa::fwd_tile_shape(s.d);
+  out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
+  out->lds_bytes = t.lds_bytes;
+  out->grid[0] = s.hq;
+  out->grid[1] = (s.max_sq + t.block_m - 1) / t.block_m;
+  out->grid[2] = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+  out->backend_index = 0;
+  out->head_dim = s.d;
+  out->flags = (s.windowed ? 1 : 0) | (s.bias ? 2 : 0) | (s.dropout ? 4 : 0) | (s.num_seqlens != 0 ? 8 : 0);
+  return FA_SUCCESS;
+}
+
+int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, int32_t kernel_slot,
+                        fa_kernel_config* out) {
+  if (out == nullptr || kernel_slot < 0 || kernel_slot > 3) return FA_ERROR_INVALID_VALUE;
+  Shape s{};
+  int be = 0;
+  int e = validate_bwd(params, FA_BWD_PARAMS_VERSION, options, &s, &be);
+  if (e != FA_SUCCESS) return e;
+  const fa::TileShape t = fa::bwd_tile_shape(s.d, kernel_slot);
+  const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+  out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
+  out->lds_bytes = t.lds_bytes;
+  const int mt = (s.max_sq + t.block_m - 1) / t.block_m, nt = (s.max_sk + t.block_n - 1) / t.block_n;
+  switch (kernel_slot) {
+    case 0: out->grid[0] = mt; out->grid[1] = s.hq; break;
+    case 1: out->grid[0] = s.hk; out->grid[1] = nt; break;
+    case 2: out->grid[0] = s.hq; out->grid[1] = mt; break;
+    default: out->grid[0] = s.hk; out->grid[1] = nt + mt * (s.hq / s.hk); break;
+  }
+  out->grid[2] = nz;
+  out->backend_index = be;
+  out->head_dim = s.d;
+  out->flags = (s.windowed ? 1 : 0) | (s.bias ? 2 : 0) | (s.dropout ? 4 : 0) | (s.num_seqlens != 0 ? 8 : 0);
+  return FA_SUCCESS;
+}
+
+int fa_debug_simulate_encoded_softmax(const fa_tensor4* r, float dropout_p, const fa_tensor0* philox_seed,
+                                      const fa_tensor0* philox_offset1, uint64_t philox_offset2,
+                                      void* hip_stream) {
+  if (r == nullptr || r->ptr == nullptr || philox_seed == nullptr || philox_offset1 == nullptr)
+    return FA_ERROR_INVALID_VALUE;
+  if (r->dtype != FA_DTYPE_FLOAT16 && r->dtype != FA_DTYPE_BFLOAT16 && r->dtype != FA_DTYPE_FLOAT32)
+    return FA_ERROR_INVALID_VALUE;
+  if (r->strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const DeviceInfo* d = device_of_stream(stream);
+  if (d == nullptr || !d->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+  fa::EncodedSoftmaxArgs a{};
+  a.r = r->ptr;
+  a.s_z = (int64_t)r->strides[0]; a.s_h = (int64_t)r->strides[1]; a.s_m = (int64_t)r->strides[2];
+  a.batch = (int)r->sizes[0]; a.heads = (int)r->sizes[1];      // attn_debug.cc:40-42
+  a.seqlen_q = (int)r->sizes[2]; a.seqlen_k = (int)r->sizes[3];
+  a.dtype = r->dtype;
+  a.drop = dropout_args(dropout_p, *philox_seed, *philox_offset1, philox_offset2);
+  return (int)fa::run_encoded_softmax(a, stream);
+}
+
+int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream,
+                const fa_options* options) {
+  Shape s{};
+  int e = validate_fwd(p, params_version, options, &s);
+  if (e != FA_SUCCESS) return e;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const DeviceInfo* dev = device_of_stream(stream);
+  if (dev == nullptr || !dev->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+
+  fa::FwdArgs a{};
+  a.q = p->Q.ptr; a.k = p->K.ptr; a.v = p->V.ptr; a.bias = p->B.ptr;
+  a.out = p->Out.ptr;
+  a.lse = static_cast<float*>(p->L.ptr);
+  a.sq = strides3(p->Q); a.sk = strides3(p->K); a.sv = strides3(p->V); a.so = strides3(p->Out);
+  if (s.bias) {
+    a.sb_z = (int64_t)p->B.strides[0]; a.sb_h = (int64_t)p->B.strides[1];
+    a.sb_m = (int64_t)p->B.strides[2]; a.sb_n = (int64_t)p->B.strides[3];
+  }
+  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk;
+  a.sm_scale = p->Sm_scale;
+  a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
+  a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
+  a.drop = dropout_args(p->dropout_p, p->philox_seed_ptr, p->philox_offset1, p->philox_offset2);
+  a.seed_out = static_cast<uint64_t*>(p->philox_seed_output.ptr);
+  a.offset_out = static_cast<uint64_t*>(p->philox_offset_output.ptr);
+  a.atomic_counter = static_cast<int32_t*>(p->persistent_atomic_counter.ptr);
+
+  const fa::TileShape t = fa::fwd_tile_shape(s.d);
+  FA_LOG(4, "attn_fwd: D=%d BLOCK_M=%d BLOCK_N=%d waves=%d lds=%d windowed=%d bias=%d dropout=%d nseq=%d",
+         s.d, t.block_m, t.block_n, t.num_waves, t.lds_bytes, (int)s.windowed, (int)s.bias,
+         (int)s.dropout, s.num_seqlens);
+  hipError_t err = run_fwd(p->Q.dtype, s.d, a, s, stream);
+  if (err != hipSuccess) return (int)err;
+  if (p->encoded_softmax.ptr != nullptr) {
+    // the forward metro chains the mask dump (modules/flash/aot/__init__.py:40-41)
+    fa_tensor4 r = p->encoded_softmax;
+    return fa_debug_simulate_encoded_softmax(&r, p->dropout_p, &p->philox_seed_ptr, &p->philox_offset1,
+                                             p->philox_offset2, hip_stream);
+  }
+  return FA_SUCCESS;
+}
+
+int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
+                const fa_options* options) {
+  Shape s{};
+  int backend = 0;
+  int e = validate_bwd(p, params_version, options, &s, &backend);
+  if (e != FA_SUCCESS) return e;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const DeviceInfo* dev = device_of_stream(stream);
+  if (dev == nullptr || !dev->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+
+  fa::BwdArgs a{};
+  a.q = p->Q.ptr; a.k = p->K.ptr; a.v = p->V.ptr; a.bias = p->B.ptr;
+  a.out = p->Out.ptr; a.dout = p->DO.ptr;
+  a.dq = p->DQ.ptr; a.dk = p->DK.ptr; a.dv = p->DV.ptr; a.db = p->DB.ptr;
+  a.lse = static_cast<const float*>(p->L.ptr);
+  a.sq = strides3(p->Q); a.sk = strides3(p->K); a.sv = strides3(p->V); a.so = strides3(p->Out);
+  a.sdo = strides3(p->DO); a.sdq = strides3(p->DQ); a.sdk = strides3(p->DK); a.sdv = strides3(p->DV);
+  if (s.bias) {
+    a.sb_z = (int64_t)p->B.strides[0]; a.sb_h = (int64_t)p->B.strides[1];
+    a.sb_m = (int64_t)p->B.strides[2]; a.sb_n = (int64_t)p->B.strides[3];
+  }
+  if (p->DB.ptr != nullptr) {
+    a.sdb_z = (int64_t)p->DB.strides[0]; a.sdb_h = (int64_t)p->DB.strides[1];
+    a.sdb_m = (int64_t)p->DB.strides[2]; a.sdb_n = (int64_t)p->DB.strides[3];
+  }
+  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk;
+  a.sm_scale = p->Sm_scale;
+  a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
+  a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
+  a.drop = dropout_args(p->dropout_p, p->philox_seed_ptr, p->philox_offset1, p->philox_offset2);
+
+  const int dt = p->Q.dtype;
+  FA_LOG(4, "attn_bwd: backend=%d D=%d windowed=%d bias=%d dropout=%d nseq=%d", backend, s.d,
+         (int)s.windowed, (int)s.bias, (int)s.dropout, s.num_seqlens);
+  hipError_t err = hipSuccess;
+  if (backend == 0) {
+    // split: delta, then dK/dV, then dQ (modules/flash/aot/__init__.py:52-59)
+    fa_lazy_tensor2* lazy = const_cast<fa_lazy_tensor2*>(&p->D);
+    fa_tensor2 delta = p->D.eager;
+    bool acquired = false;
+    if (delta.ptr == nullptr) {
+      if (lazy->acquire(lazy, &delta) != 0 || delta.ptr == nullptr) return FA_ERROR_INVALID_VALUE;
+      acquired = true;
+    }
+    a.delta = static_cast<float*>(delta.ptr);
+    err = fa::run_bwd_preprocess(dt, s.d, a, stream);
+    if (err == hipSuccess) err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+    if (err == hipSuccess) err = fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+    if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);   // attn_bwd.cc:157
+  } else {
+    a.delta = nullptr;
+    err = fa::run_bwd_fused(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+  }
+  return (int)err;
+}
+
+}  // extern "C"

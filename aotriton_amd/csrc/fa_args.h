@@ -1,0 +1,73 @@
+// Kernel argument blocks shared by the host dispatcher and the gfx950 kernels.
+// Strides are in elements; the innermost stride of every tensor is 1.
+#pragma once
+#include <stdint.h>
+
+namespace fa {
+
+struct Strides3 {   // batch, head, row
+  int64_t z, h, s;
+};
+
+struct SeqArgs {
+  const int32_t* cu_q;   // null when dense
+  const int32_t* cu_k;
+  const int32_t* ss_q;   // strided varlen only
+  const int32_t* ss_k;
+  int32_t num_seqlens;   // >0 compact/strided, <0 padded, 0 dense (attn_fwd.cc:99)
+  int32_t max_seqlen_q;
+  int32_t max_seqlen_k;
+};
+
+struct MaskArgs {
+  int32_t causal_type;   // 0 or 3
+  int32_t window_left;   // raw (sentinels allowed)
+  int32_t window_right;
+};
+
+struct DropoutArgs {
+  float p;
+  const uint64_t* seed_ptr;
+  const uint64_t* offset1_ptr;
+  uint64_t offset2;
+};
+
+struct FwdArgs {
+  const void* q; const void* k; const void* v; const void* bias;
+  void* out; float* lse;
+  Strides3 sq, sk, sv, so;
+  int64_t sb_z, sb_h, sb_m, sb_n;
+  int32_t batch, hq, hk;
+  float sm_scale;
+  SeqArgs seq;
+  MaskArgs mask;
+  DropoutArgs drop;
+  uint64_t* seed_out; uint64_t* offset_out;
+  int32_t* atomic_counter;
+  int32_t num_m_tiles;
+};
+
+struct BwdArgs {
+  const void* q; const void* k; const void* v; const void* bias;
+  const void* out; const void* dout;
+  void* dq; void* dk; void* dv; void* db;
+  const float* lse; float* delta;
+  Strides3 sq, sk, sv, so, sdo, sdq, sdk, sdv;
+  int64_t sb_z, sb_h, sb_m, sb_n;
+  int64_t sdb_z, sdb_h, sdb_m, sdb_n;
+  int32_t batch, hq, hk;
+  float sm_scale;
+  SeqArgs seq;
+  MaskArgs mask;
+  DropoutArgs drop;
+  int32_t num_m_tiles, num_n_tiles;
+};
+
+struct EncodedSoftmaxArgs {
+  void* r; int64_t s_z, s_h, s_m;
+  int32_t batch, heads, seqlen_q, seqlen_k;
+  int32_t dtype;
+  DropoutArgs drop;
+};
+
+}  // namespace fa

@@ -1,0 +1,184 @@
+// Device-side building blocks for the gfx950 flash-attention kernels:
+// MFMA wrappers, operand packing, Philox dropout, sequence bookkeeping.
+//
+// MFMA 32x32x16 register layout (wave64, lane = 32*hi + c):
+//   A operand: row  = c, k = 8*hi .. 8*hi+7   (8 x 16-bit per lane)
+//   B operand: col  = c, k = 8*hi .. 8*hi+7
+//   C/D      : col  = c, row(i) = 8*(i/4) + 4*hi + (i%4), i = 0..15
+// The contraction index is a dummy, so any permutation of k that is applied to
+// both operands is legal.  All kernels exploit that: an accumulator block is
+// re-used as an operand with k-slot (t, hi, j) <-> row 16*t + 8*(j/4) + 4*hi + (j%4),
+// and the other operand is stored in LDS in exactly that order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fa_args.h"
+#include "fa_intervals.h"
+
+namespace fa {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+template <typename T, int N>
+using vec = T __attribute__((ext_vector_type(N)));
+
+using f32x16 = vec<float, 16>;
+using f32x4 = vec<float, 4>;
+
+constexpr float kLog2e = 1.44269504089f;       // modules/flash/kernel/fwd_kernel.py:422
+constexpr float kLn2 = 0.6931471824645996f;    // modules/flash/kernel/fwd_kernel.py:610-612
+constexpr float kRcpLn2 = 1.4426950408889634f; // modules/flash/kernel/bwd_inner_dk_dv.py:185
+constexpr float kNegBig = -3.40282e+38f;       // modules/flash/kernel/fwd_kernel.py:417
+
+template <typename T> struct Traits;
+
+template <> struct Traits<bf16_t> {
+  using op_t = vec<__bf16, 8>;
+  using q4_t = vec<__bf16, 4>;
+  static __device__ __forceinline__ f32x16 mfma(op_t a, op_t b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ bf16_t cvt(float x) { return (bf16_t)x; }
+};
+
+template <> struct Traits<f16_t> {
+  using op_t = vec<_Float16, 8>;
+  using q4_t = vec<_Float16, 4>;
+  static __device__ __forceinline__ f32x16 mfma(op_t a, op_t b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f16_t cvt(float x) { return (f16_t)x; }
+};
+
+// Eight accumulator values (i = 8*half .. 8*half+7) -> one MFMA operand.
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::op_t pack8(const f32x16& s, int half) {
+  typename Traits<T>::op_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = Traits<T>::cvt(s[8 * half + j]);
+  return r;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+// Philox-4x32-10 with counter (c0, c1, 0, 0); Salmon et al. SC'11.  The
+// reference reaches it through Triton's tl.randint4x
+// (modules/flash/kernel/dropout.py:19).
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t k0, uint32_t k1,
+                                              uint32_t (&w)[4]) {
+  uint32_t c2 = 0, c3 = 0;
+#pragma unroll
+  for (int i = 0; i < 10; ++i) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  w[0] = c0; w[1] = c1; w[2] = c2; w[3] = c3;
+}
+
+struct DropoutState {
+  uint32_t k0, k1;
+  uint64_t base;     // philox_offset2 + *philox_offset1 + (z*Hq + h)*max_seqlen_q*stride
+  uint32_t stride;   // cdiv(max_seqlen_k, 4)
+  int32_t thr;
+  float scale;       // 1/(1-p)
+};
+
+__device__ __forceinline__ DropoutState make_dropout(const DropoutArgs& d, int z, int h, int hq,
+                                                     int max_seqlen_q, int max_seqlen_k) {
+  DropoutState s;
+  const uint64_t seed = d.seed_ptr ? *d.seed_ptr : 0ull;
+  uint64_t base = d.offset2;
+  if (d.offset1_ptr) base += *d.offset1_ptr;
+  s.k0 = (uint32_t)seed; s.k1 = (uint32_t)(seed >> 32);
+  s.stride = (uint32_t)((max_seqlen_k + 3) / 4);
+  // modules/flash/kernel/fwd_kernel.py:405-407
+  s.base = base + (uint64_t)(z * hq + h) * (uint64_t)max_seqlen_q * (uint64_t)s.stride;
+  s.thr = dropout_threshold(d.p);
+  s.scale = 1.0f / (1.0f - d.p);
+  return s;
+}
+
+// Keep bits of columns n0..n0+3 (n0 % 4 == 0) of row m, bit r <-> column n0+r.
+// Word order along the row is (w0, w2, w1, w3): modules/flash/kernel/dropout.py:37.
+__device__ __forceinline__ uint32_t dropout_keep4(const DropoutState& s, int m, int n0) {
+  const uint64_t ctr = s.base + (uint64_t)m * s.stride + (uint64_t)(n0 >> 2);
+  uint32_t w[4];
+  philox4x32_10((uint32_t)ctr, (uint32_t)(ctr >> 32), s.k0, s.k1, w);
+  return ((int32_t)w[0] > s.thr ? 1u : 0u) | ((int32_t)w[2] > s.thr ? 2u : 0u) |
+         ((int32_t)w[1] > s.thr ? 4u : 0u) | ((int32_t)w[3] > s.thr ? 8u : 0u);
+}
+
+// Keep bit of a single element.
+__device__ __forceinline__ bool dropout_keep1(const DropoutState& s, int m, int n) {
+  return (dropout_keep4(s, m, n & ~3) >> (n & 3)) & 1u;
+}
+
+// Per-sequence bookkeeping: modules/flash/kernel/fwd_kernel.py:243-286.
+struct SeqInfo {
+  int32_t seqlen_q, seqlen_k;
+  int32_t q_start, k_start;   // row offset inside the (packed) tensor
+  int32_t batch_index;        // index along the tensors' batch stride
+  int64_t lse_stride;         // rows per (batch, head) slab of LSE / delta
+};
+
+__device__ __forceinline__ SeqInfo get_seq(const SeqArgs& s, int z) {
+  SeqInfo r;
+  if (s.num_seqlens > 0) {
+    r.seqlen_q = s.cu_q[z + 1] - s.cu_q[z];
+    r.seqlen_k = s.cu_k[z + 1] - s.cu_k[z];
+    r.batch_index = 0;
+    if (s.ss_q != nullptr) {
+      r.q_start = s.ss_q[z];
+      r.k_start = s.ss_k[z];
+      r.lse_stride = s.ss_q[s.num_seqlens];
+    } else {
+      r.q_start = s.cu_q[z];
+      r.k_start = s.cu_k[z];
+      r.lse_stride = s.cu_q[s.num_seqlens];
+    }
+  } else if (s.num_seqlens < 0) {
+    r.seqlen_q = s.cu_q[z + 1] - s.cu_q[z];
+    r.seqlen_k = s.cu_k[z + 1] - s.cu_k[z];
+    r.q_start = 0; r.k_start = 0;
+    r.batch_index = z;
+    r.lse_stride = s.max_seqlen_q;
+  } else {
+    r.seqlen_q = s.max_seqlen_q;
+    r.seqlen_k = s.max_seqlen_k;
+    r.q_start = 0; r.k_start = 0;
+    r.batch_index = z;
+    r.lse_stride = s.max_seqlen_q;
+  }
+  return r;
+}
+
+// _lse_offset, modules/flash/kernel/fwd_kernel_inner.py:38-43
+__device__ __forceinline__ int64_t lse_offset(const SeqInfo& si, int h, int hq) {
+  return ((int64_t)si.batch_index * hq + h) * si.lse_stride + si.q_start;
+}
+
+// Heads are placed on grid.x.  Consecutive workgroup ids round-robin over the 8
+// XCDs, so remap x so that each XCD owns a contiguous range of heads and all
+// tiles of one head (and of one GQA group) share an L2.
+__device__ __forceinline__ int xcd_remap_head(int x, int num_heads) {
+  constexpr int kXcds = 8;
+  if (num_heads % kXcds != 0) return x;
+  return (x % kXcds) * (num_heads / kXcds) + x / kXcds;
+}
+
+// LDS position of key `kk` (0..BN-1) inside a transposed tile row: swaps bits 2
+// and 3 of the key index so that one 16-byte read yields the k-slot order
+// described at the top of this file.
+__device__ __forceinline__ int tr_pos(int kk) {
+  return (kk & ~12) | ((kk & 4) << 1) | ((kk & 8) >> 1);
+}
+
+}  // namespace fa

@@ -1,0 +1,371 @@
+// Forward flash-attention kernel for gfx950 (wave64, MFMA 32x32x16).
+//
+// Computes what the reference's attn_fwd does
+// (modules/flash/kernel/fwd_kernel.py:83-644, fwd_kernel_inner.py:46-287):
+// online softmax in base 2, O = softmax(S) V, LSE = (m + log2 l) ln 2.
+//
+// Work split: one workgroup = NW waves = BM = 32*NW query rows of one head; each
+// wave owns 32 rows; a lane owns ONE query row (lane%32) and half of the key
+// columns of every 32-key block, so row max / row sum are in-lane plus a single
+// cross-half exchange.  Per K/V tile of BN keys:
+//   S^T (keys x queries) = K_tile . Q^T        A = K rows from LDS, B = Q in registers
+//   O^T (d x queries)   += V_tile^T . P^T      A = V^T rows from LDS, B = P from the S^T accumulators
+// K is staged row-major in LDS; V is staged transposed ([d][key], keys permuted
+// by tr_pos) so that both A operands are single 16-byte LDS reads.
+#pragma once
+#include <type_traits>
+
+#include "fa_device.h"
+
+namespace fa {
+
+template <int D, int BN>
+struct FwdSmem {
+  static constexpr int KSTR = D + 8;     // +16 B per row: conflict-free b128 reads
+  static constexpr int VSTR = BN + 8;
+  static constexpr int K_ELEMS = BN * KSTR;
+  static constexpr int V_ELEMS = D * VSTR;
+  static constexpr int STAGES = 2;
+  static constexpr int BYTES = STAGES * (K_ELEMS + V_ELEMS) * 2;
+};
+
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
+__global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
+__attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1, D <= 128 ? 2 : 1)))
+void fwd_kernel(const FwdArgs a) {
+  using Tr = Traits<T>;
+  using op_t = typename Tr::op_t;
+  using q4_t = typename Tr::q4_t;
+  using SM = FwdSmem<D, BN>;
+  constexpr int NT = NW * 64;
+  constexpr int BM = NW * 32;
+  constexpr int KS = D / 16;    // k-steps of S^T = K Q^T
+  constexpr int MB = BN / 32;   // 32-key blocks per tile
+  constexpr int DB = D / 32;    // 32-wide blocks of the head dim
+  constexpr int TS = BN / 16;   // k-steps of O^T += V^T P^T
+  constexpr int KSTR = SM::KSTR, VSTR = SM::VSTR;
+  constexpr int K_CH = (BN * D / 8) / NT;                 // 16-byte chunks of K per thread
+  constexpr int V_BLK = (BN / 4) * (D / 8);               // 4-key x 8-d blocks of V
+  constexpr int V_PT = (V_BLK + NT - 1) / NT;
+  static_assert((BN * D / 8) % NT == 0, "K tile must split evenly");
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* Ks = reinterpret_cast<T*>(smem_raw);
+  T* Vs = Ks + SM::STAGES * SM::K_ELEMS;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
+
+  const int h = xcd_remap_head(blockIdx.x, a.hq);
+  const int mt = a.num_m_tiles - 1 - (int)blockIdx.y;   // heaviest causal tiles first
+  const int z = blockIdx.z;
+
+  if (kDropout && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0) {
+    // modules/flash/kernel/fwd_kernel.py:199-207
+    const uint64_t seed = *a.drop.seed_ptr;
+    uint64_t base = a.drop.offset2;
+    if (a.drop.offset1_ptr) base += *a.drop.offset1_ptr;
+    if (a.seed_out) *a.seed_out = seed;
+    if (a.offset_out) *a.offset_out = base;
+  }
+
+  const SeqInfo si = get_seq(a.seq, z);
+  const int q0 = mt * BM;
+  if (q0 >= si.seqlen_q) return;
+
+  Window w{0, 0};
+  if (kWindowed) w = parse_window(a.mask.causal_type, a.mask.window_left, a.mask.window_right,
+                                  si.seqlen_q, si.seqlen_k);
+  // keep row +/- window inside int32
+  w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
+  w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
+  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, BM, BN);
+
+  const int hk = h / (a.hq / a.hk);                       // fwd_kernel.py:360
+  const int row = q0 + wave * 32 + c;                     // this lane's query row
+  const bool row_ok = row < si.seqlen_q;
+  const int row_c = row_ok ? row : si.seqlen_q - 1;
+
+  T* optr = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
+            (int64_t)(si.q_start + row_c) * a.so.s;
+  float* lse_ptr = a.lse ? a.lse + lse_offset(si, h, a.hq) : nullptr;
+
+  if (br.lo > br.hi) {
+    // No visible key for any row of this tile: O = 0, LSE = +inf (fwd_kernel.py:327-355)
+    if (row_ok) {
+      q4_t zero4 = {0, 0, 0, 0};
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = zero4;
+      if (lse_ptr && hi == 0) lse_ptr[row] = __builtin_inff();
+    }
+    return;
+  }
+
+  // ---- Q rows as the B operand, resident for the whole tile ------------------
+  const T* qptr = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z +
+                  (int64_t)h * a.sq.h + (int64_t)(si.q_start + row_c) * a.sq.s;
+  op_t qreg[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const op_t*>(qptr + 16 * ks + 8 * hi);
+
+  const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
+                   (int64_t)hk * a.sk.h + (int64_t)si.k_start * a.sk.s;
+  const T* vbase = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z +
+                   (int64_t)hk * a.sv.h + (int64_t)si.k_start * a.sv.s;
+  const T* bptr = nullptr;
+  if (kBias)
+    bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)h * a.sb_h +
+           (int64_t)row_c * a.sb_m;
+
+  DropoutState ds{};
+  if (kDropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
+
+  // ---- global -> register -> LDS staging -------------------------------------
+  op_t kreg[K_CH];
+  op_t vreg[V_PT][4];
+
+  auto load_tile = [&](int j) {
+    const int n0 = j * BN;
+#pragma unroll
+    for (int i = 0; i < K_CH; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / (D / 8), cc = idx % (D / 8);
+      int n = n0 + r;
+      n = n < si.seqlen_k ? n : si.seqlen_k - 1;
+      kreg[i] = *reinterpret_cast<const op_t*>(kbase + (int64_t)n * a.sk.s + cc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < V_PT; ++i) {
+      const int blk = tid + i * NT;
+      if (V_BLK % NT == 0 || blk < V_BLK) {
+        const int kb = blk / (D / 8), dbk = blk % (D / 8);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          int n = n0 + 4 * kb + rr;
+          const bool ok = n < si.seqlen_k;
+          n = ok ? n : si.seqlen_k - 1;
+          op_t x = *reinterpret_cast<const op_t*>(vbase + (int64_t)n * a.sv.s + dbk * 8);
+          if (!ok) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = 0;   // P is 0 there, keep 0*V finite
+          }
+          vreg[i][rr] = x;
+        }
+      }
+    }
+  };
+
+  auto store_tile = [&](int stage) {
+    T* ks = Ks + stage * SM::K_ELEMS;
+    T* vs = Vs + stage * SM::V_ELEMS;
+#pragma unroll
+    for (int i = 0; i < K_CH; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / (D / 8), cc = idx % (D / 8);
+      *reinterpret_cast<op_t*>(ks + r * KSTR + cc * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_PT; ++i) {
+      const int blk = tid + i * NT;
+      if (V_BLK % NT == 0 || blk < V_BLK) {
+        const int kb = blk / (D / 8), dbk = blk % (D / 8);
+        const int pos = tr_pos(4 * kb);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          q4_t t4 = {vreg[i][0][e], vreg[i][1][e], vreg[i][2][e], vreg[i][3][e]};
+          *reinterpret_cast<q4_t*>(vs + (dbk * 8 + e) * VSTR + pos) = t4;
+        }
+      }
+    }
+  };
+
+  // ---- online softmax state --------------------------------------------------
+  f32x16 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float m_i = kNegBig;   // fwd_kernel.py:417
+  float l_i = 0.f;       // per-lane partial row sum (its half of the columns)
+  const float qk_scale = a.sm_scale * kLog2e;
+
+  auto compute = [&](int j, int stage, bool masked) {
+    const T* ks = Ks + stage * SM::K_ELEMS + c * KSTR + hi * 8;
+    const T* vs = Vs + stage * SM::V_ELEMS + c * VSTR + hi * 8;
+    f32x16 s[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[mb][i] = 0.f;
+    // S^T = K Q^T with the K operands read one k-step ahead of their MFMAs
+    op_t ka[2][MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) ka[0][mb] = *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR);
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k + 1 < KS) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          ka[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR + (k + 1) * 16);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(ka[k & 1][mb], qreg[k], s[mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // first V^T operands: in flight while the softmax runs
+    op_t va[2][DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[0][db] = *reinterpret_cast<const op_t*>(vs + db * 32 * VSTR);
+
+    // scale (+bias) (+mask), row max.  Scaling happens before the max
+    // (fwd_kernel_inner.py:166,197-205).
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[mb][i] *= qk_scale;
+    if (kBias) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          int n = j * BN + mb * 32 + 8 * (i / 4) + 4 * hi + (i % 4);
+          n = n < si.seqlen_k ? n : si.seqlen_k - 1;
+          s[mb][i] += (float)bptr[(int64_t)n * a.sb_n] * kLog2e;   // fwd_kernel_inner.py:187
+        }
+    }
+    if (masked) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int n = j * BN + mb * 32 + 8 * (i / 4) + 4 * hi + (i % 4);
+          bool vis = n < si.seqlen_k;
+          if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
+          s[mb][i] = vis ? s[mb][i] : -__builtin_inff();
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
+    mx = fmaxf(mx, xor32(mx));
+    const float m_new = fmaxf(m_i, mx);
+    const float alpha = fast_exp2(m_i - m_new);
+    float rs = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint32_t keep = 0xF;
+        if (kDropout) keep = dropout_keep4(ds, row, j * BN + mb * 32 + 8 * g + 4 * hi);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = fast_exp2(s[mb][4 * g + r] - m_new);
+          rs += p;                                     // l sums the undropped p (:213-214)
+          s[mb][4 * g + r] = (!kDropout || ((keep >> r) & 1u)) ? p : 0.f;
+        }
+      }
+    l_i = l_i * alpha + rs;
+    m_i = m_new;
+    // rescale the accumulator only when some row of this wave moved its max
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
+
+    op_t pb[TS];
+#pragma unroll
+    for (int t = 0; t < TS; ++t) pb[t] = pack8<T>(s[t / 2], t % 2);   // P cast to V's dtype (:274)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      if (t + 1 < TS) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          va[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(vs + db * 32 * VSTR + (t + 1) * 16);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] = Tr::mfma(va[t & 1][db], pb[t], o[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // ---- main loop: LDS double buffer, one barrier per tile ---------------------
+  load_tile(br.lo);
+  store_tile(0);
+  __syncthreads();
+  for (int j = br.lo; j <= br.hi; ++j) {
+    const int stage = (j - br.lo) & 1;
+    if (j < br.hi) load_tile(j + 1);
+    compute(j, stage, !br.is_full(j));
+    if (j < br.hi) store_tile(stage ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue ----------------------------------------------------------------
+  const float l = l_i + xor32(l_i);
+  const bool alive = l > 0.f;
+  float inv = alive ? 1.0f / l : 0.f;
+  if (kDropout) inv *= ds.scale;          // fwd_kernel.py:573-575
+  if (row_ok) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        q4_t t4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(o[db][4 * g + r] * inv);
+        *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
+      }
+    if (lse_ptr && hi == 0)
+      lse_ptr[row] = alive ? (m_i + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
+  }
+}
+
+// Tile table: one entry per (dtype size is irrelevant here) head dim.
+template <int D> struct FwdTile;
+template <> struct FwdTile<64>  { static constexpr int NW = 4, BN = 64; };
+template <> struct FwdTile<128> { static constexpr int NW = 4, BN = 64; };
+template <> struct FwdTile<256> { static constexpr int NW = 4, BN = 32; };
+
+template <typename T, int D, bool kWindowed, bool kBias, bool kDropout>
+hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
+  constexpr int NW = FwdTile<D>::NW, BN = FwdTile<D>::BN;
+  auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout>;
+  constexpr int smem = FwdSmem<D, BN>::BYTES;
+  if (smem > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, stream, a);
+  return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+  constexpr int BM = FwdTile<D>::NW * 32;
+  const int nseq = a.seq.num_seqlens != 0 ? (a.seq.num_seqlens < 0 ? -a.seq.num_seqlens : a.seq.num_seqlens)
+                                          : a.batch;
+  FwdArgs b = a;
+  b.num_m_tiles = (a.seq.max_seqlen_q + BM - 1) / BM;
+  dim3 grid(a.hq, b.num_m_tiles, nseq);
+  const int key = (windowed ? 4 : 0) | (bias ? 2 : 0) | (dropout ? 1 : 0);
+  switch (key) {
+    case 0: return launch_fwd_variant<T, D, false, false, false>(b, grid, stream);
+    case 1: return launch_fwd_variant<T, D, false, false, true>(b, grid, stream);
+    case 2: return launch_fwd_variant<T, D, false, true, false>(b, grid, stream);
+    case 3: return launch_fwd_variant<T, D, false, true, true>(b, grid, stream);
+    case 4: return launch_fwd_variant<T, D, true, false, false>(b, grid, stream);
+    case 5: return launch_fwd_variant<T, D, true, false, true>(b, grid, stream);
+    case 6: return launch_fwd_variant<T, D, true, true, false>(b, grid, stream);
+    default: return launch_fwd_variant<T, D, true, true, true>(b, grid, stream);
+  }
+}
+
+}  // namespace fa

@@ -1,0 +1,27 @@
+// Host-visible launchers of the gfx950 kernels (one translation unit per head dim).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "fa_args.h"
+
+namespace fa {
+
+constexpr int kDtypeF32 = 1, kDtypeF16 = 2, kDtypeBF16 = 3;
+
+struct TileShape { int block_m, block_n, num_waves, lds_bytes; };
+
+hipError_t run_fwd_d64(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_fwd_d128(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_fwd_d256(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+TileShape fwd_tile_shape(int head_dim);
+
+hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s);
+
+// backward: kernel_slot 0 = preprocess (delta), 1 = dK/dV, 2 = dQ, 3 = fused
+hipError_t run_bwd_preprocess(int dtype, int head_dim, const BwdArgs& a, hipStream_t s);
+hipError_t run_bwd_dkdv(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_bwd_dq(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_bwd_fused(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+TileShape bwd_tile_shape(int head_dim, int kernel_slot);
+
+}  // namespace fa

@@ -1,0 +1,267 @@
+/*
+ * C ABI of the MI355X (gfx950) flash-attention library.
+ *
+ * Every entry point is extern "C", takes plain pointers / sizes / strides and
+ * returns an int that carries a hipError_t value.  No C++ or torch types cross
+ * this boundary.  Each declaration names the reference interface it stands in
+ * for (paths relative to the reference tree).
+ *
+ * Conventions kept from the reference:
+ *   - tensors are views: device pointer + sizes + strides (in elements) + dtype
+ *     (include/aotriton/util.h:77-158); the last stride must be 1;
+ *   - philox seed/offset and the persistent counter are DEVICE pointers
+ *     (include/aotriton/flash.h:113-120);
+ *   - launches are asynchronous on the caller's stream, nothing is synchronised;
+ *   - the library never allocates device memory, except through the caller's
+ *     lazy-tensor callbacks (include/aotriton/util.h:224-246).
+ */
+#ifndef AOTRITON_AMD_FLASH_H
+#define AOTRITON_AMD_FLASH_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define FA_API __attribute__((visibility("default")))
+#else
+#define FA_API
+#endif
+
+/* include/aotriton/dtypes.h:12-25 -- same integer values. */
+enum fa_dtype {
+  FA_DTYPE_UNKNOWN = 0,
+  FA_DTYPE_FLOAT32 = 1,
+  FA_DTYPE_FLOAT16 = 2,
+  FA_DTYPE_BFLOAT16 = 3,
+  FA_DTYPE_INT8 = 10,
+  FA_DTYPE_INT16 = 11,
+  FA_DTYPE_INT32 = 12,
+  FA_DTYPE_INT64 = 13,
+  FA_DTYPE_UINT8 = 20,
+  FA_DTYPE_UINT16 = 21,
+  FA_DTYPE_UINT32 = 22,
+  FA_DTYPE_UINT64 = 23,
+};
+
+/* hipError_t values this library returns (include/hip/hip_runtime_api.h); the
+ * meaning of each follows python/codegen/template/shim.cc:72-100 and
+ * modules/flash/csrc/attn_fwd.cc:53-55. */
+enum fa_error {
+  FA_SUCCESS = 0,
+  FA_ERROR_INVALID_VALUE = 1,             /* null / inconsistent tensor views            */
+  FA_ERROR_INVALID_SYMBOL = 13,           /* params_version mismatch                     */
+  FA_ERROR_NO_BINARY_FOR_GPU = 209,       /* device is not gfx950                        */
+  FA_ERROR_PEER_ACCESS_UNSUPPORTED = 217, /* a forced backend cannot take this input     */
+  FA_ERROR_NOT_SUPPORTED = 801,           /* functional not built (head dim, stride, ..) */
+};
+
+/* TensorView<4|2|1|0>, include/aotriton/util.h:77-210. */
+typedef struct fa_tensor4 {
+  void* ptr;
+  uint64_t sizes[4];
+  uint64_t strides[4];
+  int32_t dtype;
+} fa_tensor4;
+
+typedef struct fa_tensor2 {
+  void* ptr;
+  uint64_t sizes[2];
+  uint64_t strides[2];
+  int32_t dtype;
+} fa_tensor2;
+
+typedef struct fa_tensor1 {
+  void* ptr;
+  uint64_t sizes[1];
+  uint64_t strides[1];
+  int32_t dtype;
+} fa_tensor1;
+
+typedef struct fa_tensor0 {
+  void* ptr;
+  int32_t dtype;
+} fa_tensor0;
+
+/* LazyTensor<2|4>, include/aotriton/util.h:224-246.  `eager.ptr != NULL` means
+ * the caller already owns the buffer; otherwise `acquire` is called at most once
+ * and only if the chosen backend reads the tensor; `dispose` is called before the
+ * entry point returns iff `acquire` ran (modules/flash/csrc/attn_bwd.cc:157-158).
+ * acquire fills *out and returns 0 on success. */
+typedef struct fa_lazy_tensor2 {
+  void* cookie;
+  int (*acquire)(struct fa_lazy_tensor2* self, fa_tensor2* out);
+  void (*dispose)(struct fa_lazy_tensor2* self);
+  fa_tensor2 eager;
+} fa_lazy_tensor2;
+
+typedef struct fa_lazy_tensor4 {
+  void* cookie;
+  int (*acquire)(struct fa_lazy_tensor4* self, fa_tensor4* out);
+  void (*dispose)(struct fa_lazy_tensor4* self);
+  fa_tensor4 eager;
+} fa_lazy_tensor4;
+
+/* attn_options, include/aotriton/flash.h:38-41.
+ * Backward backends: 0 = split (preprocess + dK/dV + dQ), 1 = fused single
+ * launch (modules/flash/aot/__init__.py:83-85).  Index 2 (prebuilt assembly
+ * backend of the reference) does not exist here and is rejected with
+ * FA_ERROR_PEER_ACCESS_UNSUPPORTED.  Forward has backend 0 only. */
+typedef struct fa_options {
+  int32_t force_backend_index; /* -1 = library's choice */
+  int32_t deterministic;       /* every backend here is deterministic */
+} fa_options;
+
+/* include/aotriton/flash.h:72-94 */
+#define FA_CAUSAL_NONE 0
+#define FA_CAUSAL_WINDOWED 3
+#define FA_WINDOW_TOP_LEFT (-2147483647)
+#define FA_WINDOW_BOTTOM_RIGHT (-2147483646)
+#define FA_VARLEN_NONE 0
+#define FA_VARLEN_COMPACT 1
+#define FA_VARLEN_PADDED 2
+#define FA_VARLEN_STRIDED 3
+
+#define FA_FWD_PARAMS_VERSION 3 /* attn_fwd_params::kVersion, flash.h:128 */
+#define FA_BWD_PARAMS_VERSION 6 /* attn_bwd_params::kVersion, flash.h:172 */
+
+/* attn_fwd_params, include/aotriton/flash.h:96-130 (same members, same order). */
+typedef struct fa_fwd_params {
+  fa_tensor4 Q;   /* (B, Hq, Sq, D)   compact varlen: (1, Hq, total_q, D) */
+  fa_tensor4 K;   /* (B, Hk, Sk, D) */
+  fa_tensor4 V;   /* (B, Hk, Sk, Dv) */
+  fa_tensor4 B;   /* additive bias (B, Hq, Sq, Sk) or null */
+  fa_tensor2 A;   /* alibi slopes: unused, must be null */
+  float Sm_scale;
+  fa_tensor2 L;   /* fp32 log-sum-exp (B*Hq, Sq) | varlen (Hq, total_q); may be null */
+  fa_tensor4 Out; /* (B, Hq, Sq, Dv) */
+  fa_tensor1 cu_seqlens_q; /* int32[num_seqlens+1] or null */
+  fa_tensor1 cu_seqlens_k;
+  int32_t Max_seqlen_q;
+  int32_t Max_seqlen_k;
+  fa_tensor1 seq_strides_q; /* strided varlen only */
+  fa_tensor1 seq_strides_k;
+  float dropout_p;
+  fa_tensor0 philox_seed_ptr; /* device uint64 */
+  fa_tensor0 philox_offset1;  /* device uint64 */
+  uint64_t philox_offset2;
+  fa_tensor0 philox_seed_output;   /* nullable */
+  fa_tensor0 philox_offset_output; /* nullable */
+  fa_tensor4 encoded_softmax;      /* nullable; filled with +-0.5 keep mask */
+  fa_tensor0 persistent_atomic_counter; /* device int32, zero on entry; optional here */
+  int8_t causal_type;
+  int8_t varlen_type;
+  int32_t window_left;
+  int32_t window_right;
+} fa_fwd_params;
+
+/* attn_bwd_params, include/aotriton/flash.h:138-174. */
+typedef struct fa_bwd_params {
+  fa_tensor4 Q;
+  fa_tensor4 K;
+  fa_tensor4 V;
+  fa_tensor4 B;
+  float Sm_scale;
+  fa_tensor4 Out;
+  fa_tensor4 DO;
+  fa_tensor4 DK;
+  fa_tensor4 DV;
+  fa_tensor4 DQ;
+  fa_tensor4 DB; /* nullable */
+  fa_tensor2 L;
+  fa_lazy_tensor2 D; /* delta; read/written by the split backend only */
+  fa_tensor1 cu_seqlens_q;
+  fa_tensor1 cu_seqlens_k;
+  int32_t Max_seqlen_q;
+  int32_t Max_seqlen_k;
+  fa_tensor1 seq_strides_q;
+  fa_tensor1 seq_strides_k;
+  float dropout_p;
+  fa_tensor0 philox_seed_ptr;
+  fa_tensor0 philox_offset1;
+  uint64_t philox_offset2;
+  int8_t causal_type;
+  int8_t varlen_type;
+  int32_t window_left;
+  int32_t window_right;
+  fa_lazy_tensor4 DQ_ACC; /* never acquired: the dQ path has a single owner per tile */
+} fa_bwd_params;
+
+/* What the compile-time tile table selected for a call; stands in for peeking at
+ * the reference's debug log (modules/flash/csrc/attn_fwd.cc:15-17). */
+typedef struct fa_kernel_config {
+  int32_t block_m;
+  int32_t block_n;
+  int32_t num_waves;
+  int32_t lds_bytes;
+  int32_t grid[3];
+  int32_t backend_index;
+  int32_t head_dim;
+  int32_t flags; /* bit0 causal/windowed, bit1 bias, bit2 dropout, bit3 varlen */
+} fa_kernel_config;
+
+/* v2::flash::check_gpu -- modules/flash/csrc/attn_check.cc:36-46.
+ * FA_SUCCESS on gfx950, FA_ERROR_NO_BINARY_FOR_GPU otherwise. */
+FA_API int fa_check_gpu(void* hip_stream);
+
+/* v3::flash::attn_fwd -- include/aotriton/flash.h:132-136,
+ * modules/flash/csrc/attn_fwd.cc:48-149. */
+FA_API int fa_attn_fwd(const fa_fwd_params* params, int32_t params_version,
+                       void* hip_stream, const fa_options* options);
+
+/* v3::flash::attn_bwd -- include/aotriton/flash.h:176-180,
+ * modules/flash/csrc/attn_bwd.cc:55-160. */
+FA_API int fa_attn_bwd(const fa_bwd_params* params, int32_t params_version,
+                       void* hip_stream, const fa_options* options);
+
+/* v2::flash::debug_simulate_encoded_softmax -- include/aotriton/flash.h:18-24,
+ * modules/flash/csrc/attn_debug.cc:30-69.  r is (B, H, max_seqlen_q, max_seqlen_k). */
+FA_API int fa_debug_simulate_encoded_softmax(const fa_tensor4* r, float dropout_p,
+                                             const fa_tensor0* philox_seed,
+                                             const fa_tensor0* philox_offset1,
+                                             uint64_t philox_offset2, void* hip_stream);
+
+/* Pure host argument checks that fa_attn_fwd / fa_attn_bwd run before any HIP
+ * call (version gate attn_fwd.cc:53-55; functional availability
+ * python/codegen/template/shim.cc:72-100). */
+FA_API int fa_validate_fwd(const fa_fwd_params* params, int32_t params_version,
+                           const fa_options* options);
+FA_API int fa_validate_bwd(const fa_bwd_params* params, int32_t params_version,
+                           const fa_options* options);
+
+/* Tile/grid the library would use (host only, num_cu = CU count to assume). */
+FA_API int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu,
+                               fa_kernel_config* out);
+FA_API int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options,
+                               int32_t kernel_slot, fa_kernel_config* out);
+
+/* K-block interval algebra used by the kernels for one Q tile (host mirror of the
+ * device function; modules/flash/kernel/masked_load_store.py:43-210).
+ * window_left/right are the raw parameters (sentinels allowed).  out[6] =
+ * {left-masked lo,hi, full lo,hi, right-masked lo,hi}, closed, empty if lo>hi. */
+FA_API int fa_tile_intervals(int32_t causal_type, int32_t window_left, int32_t window_right,
+                             int32_t start_m, int32_t seqlen_q, int32_t seqlen_k,
+                             int32_t block_m, int32_t block_n, int32_t out[6]);
+
+/* int32 keep threshold the kernels compare Philox words against
+ * (modules/flash/kernel/fwd_kernel.py:195). */
+FA_API int32_t fa_dropout_threshold(float dropout_p);
+
+/* pyaotriton.get_name_suffix -- bindings/module.cc:89-99. */
+FA_API const char* fa_get_name_suffix(void);
+FA_API const char* fa_version(void);
+
+/* v_archname / CU count -- v3src/util.cc:65-113.  buf receives e.g. "gfx950". */
+FA_API int fa_get_arch(void* hip_stream, char* buf, int32_t buflen);
+FA_API int fa_get_multiprocessor_count(void* hip_stream);
+
+/* bindings/hipruntime.cc:11-95 */
+FA_API int fa_hip_get_last_error(void);
+FA_API int fa_hip_device_synchronize(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AOTRITON_AMD_FLASH_H */

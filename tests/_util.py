@@ -1,0 +1,60 @@
+"""Shared helpers for the GPU parity tests: seeded inputs and the reference's
+tolerance model (modules/flash/tests/_common_test.py:459-495):
+    max|out - ref_hp| <= max(1e-5, fudge * max|ref_hp - ref_lp|)
+with ref_hp the oracle in fp32 and ref_lp the oracle in the input dtype.
+Fudge factors: out 3.0, dq 148, dk 48, dv 36, db 17 (_common_test.py:171-180,384-407).
+"""
+import math
+
+import numpy as np
+import torch
+
+from oracle import fa_ref, philox
+
+FUDGE = dict(out=3.0, dq=148.0, dk=48.0, dv=36.0, db=17.0)
+# the LSE has no entry in the reference's tolerance table (its tests only check
+# the known-answer case); fp32 accumulation of 16-bit products, absolute bound
+LSE_ATOL = 2e-3
+
+
+def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False):
+    g = torch.Generator(device='cpu').manual_seed(seed)
+
+    def rn(*shape, scale=1.0):
+        return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale).to(dtype).to(device)
+
+    if bshd:   # storage (B, S, H, D) viewed as (B, H, S, D): non-contiguous head stride
+        q = rn(B, Sq, Hq, D).transpose(1, 2)
+        k = rn(B, Sk, Hk, D).transpose(1, 2)
+        v = rn(B, Sk, Hk, D).transpose(1, 2)
+        do = rn(B, Sq, Hq, D).transpose(1, 2)
+    else:
+        q = rn(B, Hq, Sq, D); k = rn(B, Hk, Sk, D); v = rn(B, Hk, Sk, D); do = rn(B, Hq, Sq, D)
+    b = None
+    if bias:
+        sk8 = (Sk + 7) // 8 * 8      # rows padded to 8 then sliced (_common_test.py:197-199)
+        b = rn(B, Hq, Sq, sk8, scale=0.5)[:, :, :, :Sk]
+    return q, k, v, b, do
+
+
+def keep_mask_from_oracle(B, H, Sq, Sk, p, seed, offset, device):
+    if p <= 0:
+        return None
+    return torch.from_numpy(philox.dropout_keep_mask(B, H, Sq, Sk, p, seed, offset)).to(device)
+
+
+def ref_fwd(q, k, v, b, sm_scale, ct, wl, wr, p, keep, dtype):
+    cast = lambda t: None if t is None else t.to(dtype)
+    return fa_ref.attn_fwd_ref(cast(q), cast(k), cast(v), cast(b), sm_scale, ct, wl, wr, p, keep)
+
+
+def check(name, out, ref_hp, ref_lp, fudge, mask=None):
+    out = out.float(); ref_hp = ref_hp.float(); ref_lp = ref_lp.float()
+    if mask is not None:
+        out = out[mask]; ref_hp = ref_hp[mask]; ref_lp = ref_lp[mask]
+    assert not torch.isnan(out).any(), f'{name}: NaN in output'
+    err = (out - ref_hp).abs().max().item() if out.numel() else 0.0
+    ref_err = (ref_lp - ref_hp).abs().max().item() if out.numel() else 0.0
+    thr = max(1e-5, fudge * ref_err)
+    assert err <= thr, f'{name}: max|out-ref|={err:.3e} > {thr:.3e} (ref_lp err {ref_err:.3e}, fudge {fudge})'
+    return err, thr
