@@ -1,6 +1,824 @@
+// Backward flash-attention kernels for gfx950 (wave64, MFMA 32x32x16).
+//
+// What is computed follows the reference's split backward
+//   delta   modules/flash/kernel/bwd_preprocess.py:28-250
+//   dK, dV  modules/flash/kernel/bwd_kernel_dk_dv.py:48-417, bwd_inner_dk_dv.py:28-267
+//   dQ, dB  modules/flash/kernel/bwd_kernel_dq.py:45-389, bwd_inner_dq.py:28-215
+// and its single-launch variant modules/flash/kernel/bwd_kernel_fuse.py:49-665
+// (grid.y split into dK/dV items and dQ items, delta recomputed inline).
+// No atomics anywhere: every dK/dV tile and every dQ tile has exactly one owner.
+//
+// dK/dV item: a wave owns 32 keys (lane%32 = key), loops over Q tiles and over the
+// q-heads of its GQA group:
+//   S  (queries x keys) = Q_tile . K^T     A = Q rows from LDS,     B = K in registers
+//   dP (queries x keys) = dO_tile . V^T    A = dO rows from LDS,    B = V in registers
+//   dV^T (d x keys) += dO_tile^T . P       A = dO^T rows from LDS,  B = P from accumulators
+//   dK^T (d x keys) += Q_tile^T . dS       A = Q^T rows from LDS,   B = dS from accumulators
+// dQ item: a wave owns 32 queries (lane%32 = query), loops over K tiles:
+//   S^T  (keys x queries) = K_tile . Q^T   A = K rows from LDS,     B = Q in registers
+//   dP^T (keys x queries) = V_tile . dO^T  A = V rows from LDS,     B = dO in registers
+//   dQ^T (d x queries) += K_tile^T . dS^T  A = K^T rows from LDS,   B = dS^T from accumulators
 #pragma once
+#include <type_traits>
+
 #include "fa_device.h"
 #include "fa_kernels.h"
+
 namespace fa {
-template <int D> TileShape bwd_shape(int slot) { (void)slot; return TileShape{128, 128, 4, 0}; }
+
+// ---------------------------------------------------------------------------
+// delta = rowsum(O * dO) in fp32, same layout as LSE.
+// ---------------------------------------------------------------------------
+template <typename T, int D>
+__global__ void bwd_preprocess_kernel(const BwdArgs a) {
+  using op_t = typename Traits<T>::op_t;
+  constexpr int LPR = D / 8;               // lanes per row
+  constexpr int ROWS = 256 / LPR;
+  const int tid = threadIdx.x;
+  const int h = blockIdx.y, z = blockIdx.z;
+  const SeqInfo si = get_seq(a.seq, z);
+  const int row = blockIdx.x * ROWS + tid / LPR;
+  const int cc = tid % LPR;
+  float acc = 0.f;
+  if (row < si.seqlen_q) {
+    const int64_t ro = (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h + (int64_t)(si.q_start + row) * a.so.s;
+    const int64_t rd = (int64_t)si.batch_index * a.sdo.z + (int64_t)h * a.sdo.h + (int64_t)(si.q_start + row) * a.sdo.s;
+    const op_t o = *reinterpret_cast<const op_t*>(reinterpret_cast<const T*>(a.out) + ro + cc * 8);
+    const op_t d = *reinterpret_cast<const op_t*>(reinterpret_cast<const T*>(a.dout) + rd + cc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)o[e] * (float)d[e];
+  }
+#pragma unroll
+  for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (row < si.seqlen_q && cc == 0) a.delta[lse_offset(si, h, a.hq) + row] = acc;
 }
+
+// ---------------------------------------------------------------------------
+// Shared-memory plans
+// ---------------------------------------------------------------------------
+template <int D, int BM>
+struct DkDvSmem {   // per stage: Q, dO row-major; Q^T, dO^T transposed; L, delta
+  static constexpr int RSTR = D + 8;
+  static constexpr int TSTR = BM + 8;
+  static constexpr int ROW_ELEMS = BM * RSTR;
+  static constexpr int TR_ELEMS = D * TSTR;
+  static constexpr int STAGE_BYTES = (2 * ROW_ELEMS + 2 * TR_ELEMS) * 2 + 2 * BM * 4;
+  static constexpr int STAGES = 2;
+  static constexpr int BYTES = STAGES * STAGE_BYTES;
+};
+
+template <int D, int BN>
+struct DqSmem {     // per stage: K row-major, K^T transposed, V row-major
+  static constexpr int RSTR = D + 8;
+  static constexpr int TSTR = BN + 8;
+  static constexpr int ROW_ELEMS = BN * RSTR;
+  static constexpr int TR_ELEMS = D * TSTR;
+  static constexpr int STAGE_BYTES = (2 * ROW_ELEMS + TR_ELEMS) * 2;
+  static constexpr int STAGES = 2;
+  static constexpr int BYTES = STAGES * STAGE_BYTES;
+};
+
+template <int D> struct BwdTile;   // NW waves; dK/dV: BN = 32*NW keys x BM queries; dQ: BM = 32*NW queries x BN keys
+template <> struct BwdTile<64>  { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
+template <> struct BwdTile<128> { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
+template <> struct BwdTile<256> { static constexpr int NW = 4, DKDV_BM = 32, DQ_BN = 32; };
+
+// A 4-row x 8-column block of a row-major global tile, staged by one thread:
+// written to LDS both row-major (4 x 16 B) and transposed (8 x 8 B).
+template <typename T>
+struct Block4x8 {
+  using op_t = typename Traits<T>::op_t;
+  using q4_t = typename Traits<T>::q4_t;
+  op_t r[4];
+  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int row0, int col0, int nrows) {
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int m = row0 + rr;
+      const bool ok = m < nrows;
+      op_t x = *reinterpret_cast<const op_t*>(base + (int64_t)(ok ? m : nrows - 1) * row_stride + col0);
+      if (!ok) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = 0;
+      }
+      r[rr] = x;
+    }
+  }
+  __device__ __forceinline__ void store_rows(T* dst, int rstr, int lrow0, int col0) const {
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) *reinterpret_cast<op_t*>(dst + (lrow0 + rr) * rstr + col0) = r[rr];
+  }
+  __device__ __forceinline__ void store_transposed(T* dst, int tstr, int lrow0, int col0) const {
+    const int pos = tr_pos(lrow0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      q4_t t4 = {r[0][e], r[1][e], r[2][e], r[3][e]};
+      *reinterpret_cast<q4_t*>(dst + (col0 + e) * tstr + pos) = t4;
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// dK / dV work item
+// ---------------------------------------------------------------------------
+template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta>
+__device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const int nt, const int z,
+                                          char* smem_raw) {
+  using Tr = Traits<T>;
+  using op_t = typename Tr::op_t;
+  using q4_t = typename Tr::q4_t;
+  using SM = DkDvSmem<D, BM>;
+  constexpr int NT = NW * 64;
+  constexpr int BN = NW * 32;
+  constexpr int KS = D / 16, MB = BM / 32, DB = D / 32, TS = BM / 16;
+  constexpr int RSTR = SM::RSTR, TSTR = SM::TSTR;
+  constexpr int NBLK = (BM / 4) * (D / 8);
+  constexpr int BPT = (NBLK + NT - 1) / NT;     // 4x8 blocks per thread, per tensor
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
+
+  const SeqInfo si = get_seq(a.seq, z);
+  const int n0 = nt * BN;
+  if (n0 >= si.seqlen_k) return;
+
+  Window w{0, 0};
+  if (kWindowed) w = parse_window(a.mask.causal_type, a.mask.window_left, a.mask.window_right,
+                                  si.seqlen_q, si.seqlen_k);
+  w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
+  w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
+  // Rows are keys here, columns are queries: key n sees query m iff n - right <= m <= n + left
+  // (bwd_kernel_dk_dv.py:268-279 passes the window transposed in the same way).
+  const BlockRanges br = block_ranges(kWindowed, w.right, w.left, n0, si.seqlen_k, si.seqlen_q, BN, BM);
+
+  const int key = n0 + wave * 32 + c;
+  const bool key_ok = key < si.seqlen_k;
+  const int key_c = key_ok ? key : si.seqlen_k - 1;
+  T* dkptr = reinterpret_cast<T*>(a.dk) + (int64_t)si.batch_index * a.sdk.z + (int64_t)hk * a.sdk.h +
+             (int64_t)(si.k_start + key_c) * a.sdk.s;
+  T* dvptr = reinterpret_cast<T*>(a.dv) + (int64_t)si.batch_index * a.sdv.z + (int64_t)hk * a.sdv.h +
+             (int64_t)(si.k_start + key_c) * a.sdv.s;
+
+  if (br.lo > br.hi) {   // no query sees these keys
+    if (key_ok) {
+      q4_t zero4 = {0, 0, 0, 0};
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          *reinterpret_cast<q4_t*>(dkptr + 32 * db + 8 * g + 4 * hi) = zero4;
+          *reinterpret_cast<q4_t*>(dvptr + 32 * db + 8 * g + 4 * hi) = zero4;
+        }
+    }
+    return;
+  }
+
+  // K and V rows of this lane's key as B operands (k = head dim)
+  const T* kptr = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
+                  (int64_t)(si.k_start + key_c) * a.sk.s;
+  const T* vptr = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
+                  (int64_t)(si.k_start + key_c) * a.sv.s;
+  op_t kreg[KS], vreg[KS];
+#pragma unroll
+  for (int k = 0; k < KS; ++k) {
+    kreg[k] = *reinterpret_cast<const op_t*>(kptr + 16 * k + 8 * hi);
+    vreg[k] = *reinterpret_cast<const op_t*>(vptr + 16 * k + 8 * hi);
+  }
+
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { dk[db][i] = 0.f; dv[db][i] = 0.f; }
+
+  const int group = a.hq / a.hk;
+  const int ntq = br.hi - br.lo + 1;
+  const int total = group * ntq;
+  const float qk_scale = a.sm_scale * kLog2e;
+
+  auto stage_ptr = [&](int stage) { return smem_raw + stage * SM::STAGE_BYTES; };
+
+  // ---- staging -----------------------------------------------------------------
+  Block4x8<T> qblk[BPT], doblk[BPT];
+  float l_stage = 0.f, d_stage = 0.f;
+  float dpart[BPT][4];
+
+  auto load_tile = [&](int it) {
+    const int hq = hk * group + it / ntq;
+    const int m0 = (br.lo + it % ntq) * BM;
+    const T* qb = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)hq * a.sq.h +
+                  (int64_t)si.q_start * a.sq.s;
+    const T* dob = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
+                   (int64_t)hq * a.sdo.h + (int64_t)si.q_start * a.sdo.s;
+#pragma unroll
+    for (int b = 0; b < BPT; ++b) {
+      const int blk = tid + b * NT;
+      if (NBLK % NT == 0 || blk < NBLK) {
+        const int kb = blk / (D / 8), cb = blk % (D / 8);
+        qblk[b].load(qb, a.sq.s, m0 + 4 * kb, cb * 8, si.seqlen_q);
+        doblk[b].load(dob, a.sdo.s, m0 + 4 * kb, cb * 8, si.seqlen_q);
+        if (kInlineDelta) {
+          // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310)
+          const T* ob = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z +
+                        (int64_t)hq * a.so.h + (int64_t)si.q_start * a.so.s;
+          Block4x8<T> oblk;
+          oblk.load(ob, a.so.s, m0 + 4 * kb, cb * 8, si.seqlen_q);
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            float acc = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc += (float)oblk.r[rr][e] * (float)doblk[b].r[rr][e];
+            dpart[b][rr] = acc;
+          }
+        }
+      }
+    }
+    if (tid < BM) {
+      const int m = m0 + tid;
+      const bool ok = m < si.seqlen_q;
+      const int64_t lo = lse_offset(si, hq, a.hq) + (ok ? m : 0);
+      l_stage = ok ? a.lse[lo] * kRcpLn2 : 0.f;          // bwd_inner_dk_dv.py:185-186
+      if (!kInlineDelta) d_stage = ok ? a.delta[lo] : 0.f;
+    }
+  };
+
+  auto store_tile = [&](int stage) {
+    char* sp = stage_ptr(stage);
+    T* Qs = reinterpret_cast<T*>(sp);
+    T* dOs = Qs + SM::ROW_ELEMS;
+    T* Qt = dOs + SM::ROW_ELEMS;
+    T* dOt = Qt + SM::TR_ELEMS;
+    float* Ls = reinterpret_cast<float*>(dOt + SM::TR_ELEMS);
+    float* Ds = Ls + BM;
+#pragma unroll
+    for (int b = 0; b < BPT; ++b) {
+      const int blk = tid + b * NT;
+      if (NBLK % NT == 0 || blk < NBLK) {
+        const int kb = blk / (D / 8), cb = blk % (D / 8);
+        qblk[b].store_rows(Qs, RSTR, 4 * kb, cb * 8);
+        qblk[b].store_transposed(Qt, TSTR, 4 * kb, cb * 8);
+        doblk[b].store_rows(dOs, RSTR, 4 * kb, cb * 8);
+        doblk[b].store_transposed(dOt, TSTR, 4 * kb, cb * 8);
+        if (kInlineDelta) {
+          // the D/8 threads that share a row are consecutive lanes
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            float acc = dpart[b][rr];
+#pragma unroll
+            for (int off = (D / 8) / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+            if (cb == 0) Ds[4 * kb + rr] = acc;
+          }
+        }
+      }
+    }
+    if (tid < BM) {
+      Ls[tid] = l_stage;
+      if (!kInlineDelta) Ds[tid] = d_stage;
+    }
+  };
+
+  // ---- one (q-head, Q tile) step -----------------------------------------------
+  auto compute = [&](int it, int stage, bool masked) {
+    const int hq = hk * group + it / ntq;
+    const int m0 = (br.lo + it % ntq) * BM;
+    char* sp = stage_ptr(stage);
+    const T* Qs = reinterpret_cast<const T*>(sp) + c * RSTR + hi * 8;
+    const T* dOs = reinterpret_cast<const T*>(sp) + SM::ROW_ELEMS + c * RSTR + hi * 8;
+    const T* Qt = reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + c * TSTR + hi * 8;
+    const T* dOt = Qt + SM::TR_ELEMS;
+    const float* Ls = reinterpret_cast<const float*>(reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + 2 * SM::TR_ELEMS);
+    const float* Ds = Ls + BM;
+
+    f32x16 s[MB], dp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+
+    op_t xa[2][MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR);
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k + 1 < KS) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + (k + 1) * 16);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], kreg[k], s[mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR);
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k + 1 < KS) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + (k + 1) * 16);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], vreg[k], dp[mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // first transposed operands in flight during the elementwise part
+    op_t ta[2][DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) ta[0][db] = *reinterpret_cast<const op_t*>(dOt + db * 32 * TSTR);
+
+    DropoutState dst{};
+    if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
+    const T* bptr = nullptr;
+    if (kBias)
+      bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)hq * a.sb_h +
+             (int64_t)key_c * a.sb_n;
+
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int mloc = 32 * mb + 8 * g + 4 * hi;
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Ls + mloc);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Ds + mloc);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = 4 * g + r;
+          const int m = m0 + mloc + r;
+          float x = s[mb][i] * qk_scale;
+          if (kBias) {
+            const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
+            x += (float)bptr[(int64_t)mm * a.sb_m] * kLog2e;
+          }
+          if (masked) {
+            bool vis = (m < si.seqlen_q) & key_ok;
+            if (kWindowed) vis = vis & (key <= m + w.right) & (key >= m - w.left);
+            x = vis ? x : -__builtin_inff();
+          }
+          const float p = fast_exp2(x - l4[r]);          // bwd_inner_dk_dv.py:187-188
+          float pd = p, dpv = dp[mb][i];
+          if (kDropout) {
+            const bool keep = dropout_keep1(dst, m, key);
+            pd = keep ? p * dst.scale : 0.f;              // :200-201
+            dpv = keep ? dpv * dst.scale : 0.f;           // :239-240
+          }
+          s[mb][i] = pd;
+          dp[mb][i] = p * (dpv - d4[r]);                  // ds uses the undropped p (:242)
+        }
+      }
+
+    op_t pb[TS], sb[TS];
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      pb[t] = pack8<T>(s[t / 2], t % 2);     // p cast to dO's dtype, ds to Q's (composed_tensors.py:191-193)
+      sb[t] = pack8<T>(dp[t / 2], t % 2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      if (t + 1 < TS) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          ta[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(dOt + db * 32 * TSTR + (t + 1) * 16);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) dv[db] = Tr::mfma(ta[t & 1][db], pb[t], dv[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) ta[0][db] = *reinterpret_cast<const op_t*>(Qt + db * 32 * TSTR);
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      if (t + 1 < TS) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          ta[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(Qt + db * 32 * TSTR + (t + 1) * 16);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int it = 0; it < total; ++it) {
+    const int stage = it & 1;
+    if (it + 1 < total) load_tile(it + 1);
+    compute(it, stage, !br.is_full(br.lo + it % ntq));
+    if (it + 1 < total) store_tile(stage ^ 1);
+    __syncthreads();
+  }
+
+  if (key_ok) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        q4_t k4, v4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          k4[r] = Tr::cvt(dk[db][4 * g + r] * a.sm_scale);   // bwd_kernel_dk_dv.py:387-389
+          v4[r] = Tr::cvt(dv[db][4 * g + r]);
+        }
+        *reinterpret_cast<q4_t*>(dkptr + 32 * db + 8 * g + 4 * hi) = k4;
+        *reinterpret_cast<q4_t*>(dvptr + 32 * db + 8 * g + 4 * hi) = v4;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dQ (+dB) work item
+// ---------------------------------------------------------------------------
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta>
+__device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int mt, const int z,
+                                        char* smem_raw) {
+  using Tr = Traits<T>;
+  using op_t = typename Tr::op_t;
+  using q4_t = typename Tr::q4_t;
+  using SM = DqSmem<D, BN>;
+  constexpr int NT = NW * 64;
+  constexpr int BM = NW * 32;
+  constexpr int KS = D / 16, MB = BN / 32, DB = D / 32, TS = BN / 16;
+  constexpr int RSTR = SM::RSTR, TSTR = SM::TSTR;
+  constexpr int NBLK = (BN / 4) * (D / 8);
+  constexpr int BPT = (NBLK + NT - 1) / NT;
+  constexpr int V_CH = (BN * D / 8) / NT;
+  static_assert((BN * D / 8) % NT == 0, "V tile must split evenly");
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
+
+  const SeqInfo si = get_seq(a.seq, z);
+  const int q0 = mt * BM;
+  if (q0 >= si.seqlen_q) return;
+
+  Window w{0, 0};
+  if (kWindowed) w = parse_window(a.mask.causal_type, a.mask.window_left, a.mask.window_right,
+                                  si.seqlen_q, si.seqlen_k);
+  w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
+  w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
+  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, BM, BN);
+
+  const int hk = h / (a.hq / a.hk);
+  const int row = q0 + wave * 32 + c;
+  const bool row_ok = row < si.seqlen_q;
+  const int row_c = row_ok ? row : si.seqlen_q - 1;
+
+  T* dqptr = reinterpret_cast<T*>(a.dq) + (int64_t)si.batch_index * a.sdq.z + (int64_t)h * a.sdq.h +
+             (int64_t)(si.q_start + row_c) * a.sdq.s;
+  T* dbptr = nullptr;
+  if (kBias && a.db != nullptr)
+    dbptr = reinterpret_cast<T*>(a.db) + (int64_t)si.batch_index * a.sdb_z + (int64_t)h * a.sdb_h +
+            (int64_t)row_c * a.sdb_m;
+  const int nkt = (si.seqlen_k + BN - 1) / BN;
+
+  // dB of K tiles that are never visited is zero
+  auto zero_db = [&](int j_from, int j_to) {
+    if (!(kBias && dbptr != nullptr && row_ok)) return;
+    for (int j = j_from; j < j_to; ++j)
+      for (int i = hi; i < BN; i += 2) {
+        const int n = j * BN + i;
+        if (n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(0.f);
+      }
+  };
+
+  if (br.lo > br.hi) {
+    if (row_ok) {
+      q4_t zero4 = {0, 0, 0, 0};
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = zero4;
+    }
+    zero_db(0, nkt);
+    return;
+  }
+
+  const T* qptr = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
+                  (int64_t)(si.q_start + row_c) * a.sq.s;
+  const T* doptr = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
+                   (int64_t)h * a.sdo.h + (int64_t)(si.q_start + row_c) * a.sdo.s;
+  op_t qreg[KS], doreg[KS];
+#pragma unroll
+  for (int k = 0; k < KS; ++k) {
+    qreg[k] = *reinterpret_cast<const op_t*>(qptr + 16 * k + 8 * hi);
+    doreg[k] = *reinterpret_cast<const op_t*>(doptr + 16 * k + 8 * hi);
+  }
+  const int64_t lo = lse_offset(si, h, a.hq) + row_c;
+  const float l_row = a.lse[lo] * kRcpLn2;               // bwd_kernel_dq.py:305
+  float d_row;
+  if (kInlineDelta) {
+    const T* optr = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z +
+                    (int64_t)h * a.so.h + (int64_t)(si.q_start + row_c) * a.so.s;
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      const op_t o8 = *reinterpret_cast<const op_t*>(optr + 16 * k + 8 * hi);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += (float)o8[e] * (float)doreg[k][e];
+    }
+    d_row = acc + xor32(acc);
+  } else {
+    d_row = a.delta[lo];
+  }
+
+  const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
+                   (int64_t)si.k_start * a.sk.s;
+  const T* vbase = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
+                   (int64_t)si.k_start * a.sv.s;
+  const T* bptr = nullptr;
+  if (kBias)
+    bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)h * a.sb_h +
+           (int64_t)row_c * a.sb_m;
+  DropoutState dst{};
+  if (kDropout) dst = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
+
+  f32x16 dq[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dq[db][i] = 0.f;
+  const float qk_scale = a.sm_scale * kLog2e;
+
+  Block4x8<T> kblk[BPT];
+  op_t vch[V_CH];
+
+  auto load_tile = [&](int j) {
+    const int nn0 = j * BN;
+#pragma unroll
+    for (int b = 0; b < BPT; ++b) {
+      const int blk = tid + b * NT;
+      if (NBLK % NT == 0 || blk < NBLK) {
+        const int kb = blk / (D / 8), cb = blk % (D / 8);
+        kblk[b].load(kbase, a.sk.s, nn0 + 4 * kb, cb * 8, si.seqlen_k);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < V_CH; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / (D / 8), cc = idx % (D / 8);
+      int n = nn0 + r;
+      n = n < si.seqlen_k ? n : si.seqlen_k - 1;
+      vch[i] = *reinterpret_cast<const op_t*>(vbase + (int64_t)n * a.sv.s + cc * 8);
+    }
+  };
+  auto store_tile = [&](int stage) {
+    T* Ks = reinterpret_cast<T*>(smem_raw + stage * SM::STAGE_BYTES);
+    T* Vs = Ks + SM::ROW_ELEMS;
+    T* Kt = Vs + SM::ROW_ELEMS;
+#pragma unroll
+    for (int b = 0; b < BPT; ++b) {
+      const int blk = tid + b * NT;
+      if (NBLK % NT == 0 || blk < NBLK) {
+        const int kb = blk / (D / 8), cb = blk % (D / 8);
+        kblk[b].store_rows(Ks, RSTR, 4 * kb, cb * 8);
+        kblk[b].store_transposed(Kt, TSTR, 4 * kb, cb * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < V_CH; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / (D / 8), cc = idx % (D / 8);
+      *reinterpret_cast<op_t*>(Vs + r * RSTR + cc * 8) = vch[i];
+    }
+  };
+
+  auto compute = [&](int j, int stage, bool masked) {
+    const T* Ks = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + c * RSTR + hi * 8;
+    const T* Vs = Ks + SM::ROW_ELEMS;
+    const T* Kt = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + 2 * SM::ROW_ELEMS +
+                  c * TSTR + hi * 8;
+    f32x16 s[MB], dp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+    op_t xa[2][MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR);
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k + 1 < KS) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + (k + 1) * 16);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], qreg[k], s[mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR);
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k + 1 < KS) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + (k + 1) * 16);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], doreg[k], dp[mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    op_t ta[2][DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) ta[0][db] = *reinterpret_cast<const op_t*>(Kt + db * 32 * TSTR);
+
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int nb = j * BN + 32 * mb + 8 * g + 4 * hi;
+        uint32_t keep = 0xF;
+        if (kDropout) keep = dropout_keep4(dst, row, nb);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = 4 * g + r;
+          const int n = nb + r;
+          float x = s[mb][i] * qk_scale;
+          if (kBias) {
+            const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
+            x += (float)bptr[(int64_t)nn * a.sb_n] * kLog2e;
+          }
+          if (masked) {
+            bool vis = n < si.seqlen_k;
+            if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
+            x = vis ? x : -__builtin_inff();
+          }
+          const float p = fast_exp2(x - l_row);
+          float dpv = dp[mb][i];
+          if (kDropout) dpv = ((keep >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
+          const float dsv = p * (dpv - d_row);
+          dp[mb][i] = dsv;
+          if (kBias && dbptr != nullptr && row_ok && n < si.seqlen_k)
+            dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);                      // bwd_inner_dq.py:200-204
+        }
+      }
+    op_t sb[TS];
+#pragma unroll
+    for (int t = 0; t < TS; ++t) sb[t] = pack8<T>(dp[t / 2], t % 2);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      if (t + 1 < TS) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          ta[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(Kt + db * 32 * TSTR + (t + 1) * 16);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) dq[db] = Tr::mfma(ta[t & 1][db], sb[t], dq[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  load_tile(br.lo);
+  store_tile(0);
+  __syncthreads();
+  for (int j = br.lo; j <= br.hi; ++j) {
+    const int stage = (j - br.lo) & 1;
+    if (j < br.hi) load_tile(j + 1);
+    compute(j, stage, !br.is_full(j));
+    if (j < br.hi) store_tile(stage ^ 1);
+    __syncthreads();
+  }
+
+  if (row_ok) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        q4_t t4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(dq[db][4 * g + r] * a.sm_scale);   // bwd_kernel_dq.py:374-376
+        *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = t4;
+      }
+  }
+  zero_db(0, br.lo);
+  zero_db(br.hi + 1, nkt);
+}
+
+// ---------------------------------------------------------------------------
+// Kernels
+// ---------------------------------------------------------------------------
+template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout>
+__global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
+void bwd_dkdv_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  const int hk = xcd_remap_head(blockIdx.x, a.hk);
+  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false>(a, hk, blockIdx.y, blockIdx.z, smem_raw);
+}
+
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
+__global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
+void bwd_dq_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  const int h = xcd_remap_head(blockIdx.x, a.hq);
+  const int mt = a.num_m_tiles - 1 - (int)blockIdx.y;
+  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, h, mt, blockIdx.z, smem_raw);
+}
+
+// grid.y = num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
+// (modules/flash/csrc/attn_bwd_fused.cc:13-22, bwd_kernel_fuse.py:107-118).
+template <typename T, int D, int NW, int BM, int BN, bool kWindowed, bool kBias, bool kDropout>
+__global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
+void bwd_fused_kernel(const BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  const int hk = xcd_remap_head(blockIdx.x, a.hk);
+  const int item = blockIdx.y;
+  if (item < a.num_n_tiles) {
+    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true>(a, hk, item, blockIdx.z, smem_raw);
+  } else {
+    const int t = item - a.num_n_tiles;
+    const int group = a.hq / a.hk;
+    const int h = hk * group + t / a.num_m_tiles;
+    const int mt = a.num_m_tiles - 1 - t % a.num_m_tiles;
+    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true>(a, h, mt, blockIdx.z, smem_raw);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host launchers
+// ---------------------------------------------------------------------------
+inline int bwd_nseq(const BwdArgs& a) {
+  return a.seq.num_seqlens != 0 ? (a.seq.num_seqlens < 0 ? -a.seq.num_seqlens : a.seq.num_seqlens) : a.batch;
+}
+
+template <typename K>
+hipError_t launch_with_lds(K kern, dim3 grid, int nthreads, int smem, hipStream_t stream, const BwdArgs& a) {
+  if (smem > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(nthreads), smem, stream, a);
+  return hipGetLastError();
+}
+
+#define FA_BWD_SWITCH(CALL)                                            \
+  switch ((windowed ? 4 : 0) | (bias ? 2 : 0) | (dropout ? 1 : 0)) {   \
+    case 0: return CALL(false, false, false);                          \
+    case 1: return CALL(false, false, true);                           \
+    case 2: return CALL(false, true, false);                           \
+    case 3: return CALL(false, true, true);                            \
+    case 4: return CALL(true, false, false);                           \
+    case 5: return CALL(true, false, true);                            \
+    case 6: return CALL(true, true, false);                            \
+    default: return CALL(true, true, true);                            \
+  }
+
+template <typename T, int D>
+hipError_t launch_bwd_preprocess(const BwdArgs& a, hipStream_t stream) {
+  constexpr int ROWS = 256 / (D / 8);
+  dim3 grid((a.seq.max_seqlen_q + ROWS - 1) / ROWS, a.hq, bwd_nseq(a));
+  hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), grid, dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+  constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = NW * 32;
+  BwdArgs a = a0;
+  a.num_n_tiles = (a.seq.max_seqlen_k + BN - 1) / BN;
+  dim3 grid(a.hk, a.num_n_tiles, bwd_nseq(a));
+#define FA_CALL(W, B, P) launch_with_lds(bwd_dkdv_kernel<T, D, NW, BM, W, B, P>, grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
+  FA_BWD_SWITCH(FA_CALL)
+#undef FA_CALL
+}
+
+template <typename T, int D>
+hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+  constexpr int NW = BwdTile<D>::NW, BN = BwdTile<D>::DQ_BN, BM = NW * 32;
+  BwdArgs a = a0;
+  a.num_m_tiles = (a.seq.max_seqlen_q + BM - 1) / BM;
+  dim3 grid(a.hq, a.num_m_tiles, bwd_nseq(a));
+#define FA_CALL(W, B, P) launch_with_lds(bwd_dq_kernel<T, D, NW, BN, W, B, P>, grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
+  FA_BWD_SWITCH(FA_CALL)
+#undef FA_CALL
+}
+
+template <typename T, int D>
+hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+  constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = BwdTile<D>::DQ_BN;
+  constexpr int smem = DkDvSmem<D, BM>::BYTES > DqSmem<D, BN>::BYTES ? DkDvSmem<D, BM>::BYTES : DqSmem<D, BN>::BYTES;
+  BwdArgs a = a0;
+  a.num_n_tiles = (a.seq.max_seqlen_k + NW * 32 - 1) / (NW * 32);
+  a.num_m_tiles = (a.seq.max_seqlen_q + NW * 32 - 1) / (NW * 32);
+  dim3 grid(a.hk, a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk), bwd_nseq(a));
+#define FA_CALL(W, B, P) launch_with_lds(bwd_fused_kernel<T, D, NW, BM, BN, W, B, P>, grid, NW * 64, smem, stream, a)
+  FA_BWD_SWITCH(FA_CALL)
+#undef FA_CALL
+}
+
+template <int D> TileShape bwd_shape(int slot) {
+  constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = BwdTile<D>::DQ_BN;
+  constexpr int s1 = DkDvSmem<D, BM>::BYTES, s2 = DqSmem<D, BN>::BYTES;
+  switch (slot) {
+    case 0: return TileShape{256 / (D / 8), 0, 4, 0};
+    case 1: return TileShape{BM, NW * 32, NW, s1};
+    case 2: return TileShape{NW * 32, BN, NW, s2};
+    default: return TileShape{NW * 32, NW * 32, NW, s1 > s2 ? s1 : s2};
+  }
+}
+
+}  // namespace fa

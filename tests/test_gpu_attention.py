@@ -1,0 +1,96 @@
+"""GPU parity tests: HIP kernels (through the C ABI) against the CPU-restated
+oracle run in fp32 on the same seeded inputs.  Tolerances are the reference's
+(tests/_util.py).  Case grid mirrors the reference's default `test_fast` grid
+(modules/flash/tests/test_backward.py:34-49) at the built head dims: ragged Sq/Sk,
+GQA, BSHD strides, causal on/off, dropout on/off, fp16/bf16."""
+import math
+
+import pytest
+import torch
+
+from _util import FUDGE, LSE_ATOL, check, keep_mask_from_oracle, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+DEV = 'cuda'
+
+
+def _run_case(B, Hq, Hk, Sq, Sk, D, dtype, causal, dropout_p=0.0, bias=False, bshd=False,
+              bwd_backend=-1, sm_scale=None, seed=0):
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    q, k, v, b, do = make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, DEV, seed=seed, bias=bias, bshd=bshd)
+    sm_scale = 1.0 / math.sqrt(D) if sm_scale is None else sm_scale
+    ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=bwd_backend)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    bg = b.clone().requires_grad_() if b is not None else None
+    o, _, L = attention(qg, kg, vg, bg, causal, sm_scale, dropout_p, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    assert flash.hipGetLastError() == flash.hipError_t.hipSuccess
+
+    ct, wl, wr = flash.translate_causal(causal)
+    keep = keep_mask_from_oracle(B, Hq, Sq, Sk, dropout_p, ext.philox_seed,
+                                 ext.philox_offset1 + ext.philox_offset2, DEV)
+    f32 = lambda t: None if t is None else t.float()
+    ro, rl, _ = fa_ref.attn_fwd_ref(f32(q), f32(k), f32(v), f32(b), sm_scale, ct, wl, wr, dropout_p, keep)
+    lo, ll, _ = fa_ref.attn_fwd_ref(q, k, v, b, sm_scale, ct, wl, wr, dropout_p, keep)
+    live = torch.isfinite(rl)
+    check('out', o, ro, lo, FUDGE['out'])
+    Lv = L.view(B, Hq, Sq)
+    assert torch.equal(torch.isinf(Lv), ~live), 'LSE must be +inf exactly on rows with no visible key'
+    assert (Lv[live] - rl[live]).abs().max().item() <= LSE_ATOL
+    rg = fa_ref.attn_bwd_ref(f32(q), f32(k), f32(v), f32(b), sm_scale, ro, f32(do), rl, ct, wl, wr, dropout_p, keep)
+    lg = fa_ref.attn_bwd_ref(q, k, v, b, sm_scale, lo, do, ll.to(q.dtype).float().to(q.dtype), ct, wl, wr,
+                             dropout_p, keep)
+    check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
+    check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
+    check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
+    if b is not None:
+        check('db', bg.grad, rg[3], lg[3], FUDGE['db'])
+
+
+DTYPES = [torch.bfloat16, torch.float16]
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('D', [64, 128, 256])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_dense_square(dtype, D, causal, backend):
+    _run_case(2, 4, 4, 256, 256, D, dtype, causal, bwd_backend=backend)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('D', [64, 128, 256])
+@pytest.mark.parametrize('sq,sk', [(11, 31), (523, 337), (203, 1063), (128, 77)])
+@pytest.mark.parametrize('causal', [False, True])
+def test_ragged_gqa_bshd(dtype, D, sq, sk, causal):
+    # B=3, heads (10,2), BSHD storage: the reference's default grid
+    _run_case(3, 10, 2, sq, sk, D, dtype, causal, bshd=True, sm_scale=1.0 / D)
+
+
+@pytest.mark.parametrize('D', [64, 128])
+@pytest.mark.parametrize('causal', [False, True, (17, 5), 2])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_dropout(D, causal, backend):
+    _run_case(2, 5, 5, 197, 223, D, torch.float16, causal, dropout_p=0.5, bwd_backend=backend)
+
+
+@pytest.mark.parametrize('D', [64, 128, 256])
+@pytest.mark.parametrize('causal', [False, (40, 0), True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_bias_and_db(D, causal, backend):
+    _run_case(2, 3, 3, 150, 201, D, torch.float16, causal, bias=True, bwd_backend=backend)
+
+
+def test_window_bias_dropout_small_config5():
+    # BASELINE config 5 at a size the oracle handles: window (left, 0) + bias + dropout 0.1
+    _run_case(1, 2, 2, 384, 384, 256, torch.float16, (100, 0), dropout_p=0.1, bias=True)
+
+
+@pytest.mark.parametrize('causal', [1, 2])
+def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
+    # rows with no visible key: O = 0, LSE = +inf, gradients finite
+    _run_case(2, 2, 2, 300, 140, 128, torch.bfloat16, causal)
