@@ -420,10 +420,18 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
   return FA_SUCCESS;
 }
 
-int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
-                const fa_options* options) {
+// kernel_slot < 0: the whole backward of the chosen backend; otherwise only that
+// kernel (0 delta, 1 dK/dV, 2 dQ, 3 fused).
+static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
+                         const fa_options* options, int kernel_slot) {
   Shape s{};
   int backend = 0;
+  fa_options forced{};
+  if (kernel_slot >= 0) {
+    forced.force_backend_index = kernel_slot == 3 ? 1 : 0;
+    forced.deterministic = 0;
+    options = &forced;
+  }
   int e = validate_bwd(p, params_version, options, &s, &backend);
   if (e != FA_SUCCESS) return e;
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
@@ -452,8 +460,8 @@ int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream
   a.drop = dropout_args(p->dropout_p, p->philox_seed_ptr, p->philox_offset1, p->philox_offset2);
 
   const int dt = p->Q.dtype;
-  FA_LOG(4, "attn_bwd: backend=%d D=%d windowed=%d bias=%d dropout=%d nseq=%d", backend, s.d,
-         (int)s.windowed, (int)s.bias, (int)s.dropout, s.num_seqlens);
+  FA_LOG(4, "attn_bwd: backend=%d slot=%d D=%d windowed=%d bias=%d dropout=%d nseq=%d", backend,
+         kernel_slot, s.d, (int)s.windowed, (int)s.bias, (int)s.dropout, s.num_seqlens);
   hipError_t err = hipSuccess;
   if (backend == 0) {
     // split: delta, then dK/dV, then dQ (modules/flash/aot/__init__.py:52-59)
@@ -465,15 +473,28 @@ int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream
       acquired = true;
     }
     a.delta = static_cast<float*>(delta.ptr);
-    err = fa::run_bwd_preprocess(dt, s.d, a, stream);
-    if (err == hipSuccess) err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
-    if (err == hipSuccess) err = fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+    if (kernel_slot < 0 || kernel_slot == 0) err = fa::run_bwd_preprocess(dt, s.d, a, stream);
+    if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 1))
+      err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+    if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 2))
+      err = fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);   // attn_bwd.cc:157
   } else {
     a.delta = nullptr;
     err = fa::run_bwd_fused(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
   }
   return (int)err;
+}
+
+int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
+                const fa_options* options) {
+  return attn_bwd_impl(p, params_version, hip_stream, options, -1);
+}
+
+int fa_attn_bwd_kernel(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
+                       int32_t kernel_slot) {
+  if (kernel_slot < 0 || kernel_slot > 3) return FA_ERROR_INVALID_VALUE;
+  return attn_bwd_impl(p, params_version, hip_stream, nullptr, kernel_slot);
 }
 
 }  // extern "C"

@@ -129,6 +129,14 @@ def attn_bwd(params, params_version, stream, options=None):
     return hipError_t(lib.fa_attn_bwd(ctypes.byref(c), int(params_version), stream.native() or None, optp))
 
 
+def attn_bwd_kernel(params, params_version, stream, kernel_slot):
+    """Launch one backward kernel only (0 delta, 1 dK/dV, 2 dQ, 3 fused)."""
+    from .. import hipError_t
+    c = params.to_c()
+    return hipError_t(lib.fa_attn_bwd_kernel(ctypes.byref(c), int(params_version),
+                                             stream.native() or None, int(kernel_slot)))
+
+
 def validate_fwd(params, params_version, options=None):
     from .. import hipError_t
     c = params.to_c()

@@ -216,6 +216,14 @@ FA_API int fa_attn_fwd(const fa_fwd_params* params, int32_t params_version,
 FA_API int fa_attn_bwd(const fa_bwd_params* params, int32_t params_version,
                        void* hip_stream, const fa_options* options);
 
+/* One kernel of the backward only: kernel_slot 0 = delta (bwd_preprocess), 1 = dK/dV,
+ * 2 = dQ, 3 = fused.  Slots 0-2 need an eager delta buffer in params->D.  Stands in
+ * for the per-kernel selection of the reference's tuning interface
+ * (attn_options::KernelSlot, include/aotriton/flash.h:46-60; include/aotriton/cpp_tune.h)
+ * and is what the benchmark uses to time kernels one at a time. */
+FA_API int fa_attn_bwd_kernel(const fa_bwd_params* params, int32_t params_version,
+                              void* hip_stream, int32_t kernel_slot);
+
 /* v2::flash::debug_simulate_encoded_softmax -- include/aotriton/flash.h:18-24,
  * modules/flash/csrc/attn_debug.cc:30-69.  r is (B, H, max_seqlen_q, max_seqlen_k). */
 FA_API int fa_debug_simulate_encoded_softmax(const fa_tensor4* r, float dropout_p,

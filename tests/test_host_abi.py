@@ -1,0 +1,188 @@
+"""CPU tests of the C ABI: the library loads, exports every declared symbol, and
+its pure-host argument checks / tile algebra behave as the header says.  No
+compute call is made."""
+import ctypes
+import os
+import random
+import re
+
+import pytest
+import torch
+
+from oracle import intervals as iv
+from oracle import philox
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib():
+    from aotriton_amd import _lib
+    return _lib
+
+
+def test_exports_every_declared_symbol():
+    L = _lib()
+    hdr = open(os.path.join(ROOT, 'include', 'aotriton_amd', 'flash.h')).read()
+    declared = set(re.findall(r'FA_API\s+[\w\s\*]+?\b(fa_\w+)\s*\(', hdr))
+    assert declared, 'no declarations parsed'
+    assert declared == set(L.SYMBOLS), (declared ^ set(L.SYMBOLS))
+    for name in declared:
+        assert getattr(L.lib, name) is not None
+
+
+def test_struct_layout_matches_header_order():
+    L = _lib()
+    names = [f[0] for f in L.fa_fwd_params._fields_]
+    # attn_fwd_params member order, include/aotriton/flash.h:96-126 of the reference
+    assert names == ['Q', 'K', 'V', 'B', 'A', 'Sm_scale', 'L', 'Out', 'cu_seqlens_q', 'cu_seqlens_k',
+                     'Max_seqlen_q', 'Max_seqlen_k', 'seq_strides_q', 'seq_strides_k', 'dropout_p',
+                     'philox_seed_ptr', 'philox_offset1', 'philox_offset2', 'philox_seed_output',
+                     'philox_offset_output', 'encoded_softmax', 'persistent_atomic_counter',
+                     'causal_type', 'varlen_type', 'window_left', 'window_right']
+    assert ctypes.sizeof(L.fa_tensor4) == 80 and ctypes.sizeof(L.fa_tensor0) == 16
+
+
+def test_suffix_and_threshold():
+    from aotriton_amd import flash
+    assert flash.get_name_suffix() != ''          # aotriton_flash.py:66-69 requires a suffix
+    L = _lib()
+    for p in (0.1, 0.2, 0.5, 0.0, 0.999):
+        assert L.lib.fa_dropout_threshold(p) == philox.idropout_p(p)
+    assert L.lib.fa_dropout_threshold(0.1) == -1717986944
+
+
+def test_translate_causal_table():
+    from aotriton_amd.flash import translate_causal, CausalType, WindowValue
+    assert translate_causal(False) == (0, 0, 0)
+    assert translate_causal(True) == (3, WindowValue.TOP_LEFT_ALIGNED, WindowValue.TOP_LEFT_ALIGNED)
+    assert translate_causal((5, 7)) == (3, 5, 7)
+    assert translate_causal(CausalType.TOP_LEFT) == (3, -2147483647, -2147483647)
+    assert translate_causal(CausalType.BOTTOM_RIGHT) == (3, -2147483646, -2147483646)
+    assert translate_causal(CausalType.NONE) == (0, 0, 0)
+
+
+def test_mk_aotensor_ranks():
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton import T0, T1, T2, T4, DType
+    q = torch.zeros(2, 3, 4, 8, dtype=torch.float16)
+    v = flash.mk_aotensor(q)
+    assert isinstance(v, T4) and v.sizes == [2, 3, 4, 8] and v.strides == [96, 32, 8, 1] and v.dtype == DType.kFloat16
+    assert isinstance(flash.mk_aotensor(torch.zeros(5, dtype=torch.int32)), T1)
+    assert isinstance(flash.mk_aotensor(torch.zeros(2, 5)), T2)
+    s = flash.mk_aotensor(torch.zeros(1, dtype=torch.uint64))
+    assert isinstance(s, T0) and s.dtype == DType.kUInt64
+    e = flash.mk_aotensor(torch.empty(0, dtype=torch.int32))
+    assert isinstance(e, T0) and not e
+    n = flash.mk_aotensor(None, if_empty_then_like=q)
+    assert isinstance(n, T4) and not n and n.dtype == DType.kFloat16
+    with pytest.raises(AssertionError):
+        flash.mk_aotensor(q.transpose(2, 3))
+    assert flash.cast_dtype(torch.bfloat16) == DType.kBFloat16
+    assert flash.cast_dtype(torch.float32) == DType.kFloat32
+
+
+def _fwd_params(D=128, dtype=torch.bfloat16, Hq=4, Hk=2, Sq=64, Sk=80, B=2):
+    """Views over CPU tensors: fine for the pure-host checks (nothing is launched)."""
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton.v3.flash import attn_fwd_params
+    keep = dict(q=torch.zeros(B, Hq, Sq, D, dtype=dtype), k=torch.zeros(B, Hk, Sk, D, dtype=dtype),
+                v=torch.zeros(B, Hk, Sk, D, dtype=dtype), o=torch.zeros(B, Hq, Sq, D, dtype=dtype),
+                M=torch.zeros(B * Hq, Sq))
+    p = attn_fwd_params()
+    p.Q = flash.mk_aotensor(keep['q']); p.K = flash.mk_aotensor(keep['k']); p.V = flash.mk_aotensor(keep['v'])
+    p.Out = flash.mk_aotensor(keep['o']); p.L = flash.mk_aotensor(keep['M'])
+    p.Sm_scale = 0.1
+    return p, keep
+
+
+def test_validate_fwd_error_contract():
+    from aotriton_amd.pyaotriton import hipError_t as E, T4, T2, DType
+    from aotriton_amd.pyaotriton.v3.flash import validate_fwd, attn_fwd_params, attn_options, query_fwd_config
+    p, keep = _fwd_params()
+    assert validate_fwd(p, attn_fwd_params.kVersion) == E.hipSuccess
+    assert validate_fwd(p, 2) == E.hipErrorInvalidSymbol                       # version gate
+    p2, k2 = _fwd_params(D=96)
+    assert validate_fwd(p2, 3) == E.hipErrorNotSupported                       # head dim not built
+    p3, k3 = _fwd_params(dtype=torch.float32)
+    assert validate_fwd(p3, 3) == E.hipErrorNotSupported                       # fp32 kernels not built
+    p4, k4 = _fwd_params(Hq=5, Hk=2)
+    assert validate_fwd(p4, 3) == E.hipErrorInvalidValue                       # heads not divisible
+    p.Q = T4(0, [0] * 4, [0] * 4, DType.kBFloat16)
+    assert validate_fwd(p, 3) == E.hipErrorInvalidValue                        # null Q
+    p, keep = _fwd_params()
+    p.causal_type = 1
+    assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # only 0 and 3 exist
+    p.causal_type = 3
+    p.dropout_p = 0.5
+    assert validate_fwd(p, 3) == E.hipErrorInvalidValue                        # dropout without a seed
+    p.dropout_p = 0.0
+    opt = attn_options(); opt.force_backend_index = 1
+    assert validate_fwd(p, 3, opt) == E.hipErrorPeerAccessUnsupported          # forced unknown backend
+    p.A = T2(1234, [1, 1], [1, 1], DType.kFloat32)
+    assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # alibi
+    p, keep = _fwd_params()
+    err, cfg = query_fwd_config(p)
+    assert err == E.hipSuccess and cfg.block_m == 128 and cfg.head_dim == 128
+    assert list(cfg.grid) == [4, 1, 2]
+
+
+def test_validate_bwd_error_contract():
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton import hipError_t as E
+    from aotriton_amd.pyaotriton.v3.flash import validate_bwd, attn_bwd_params, attn_options
+    B, Hq, Hk, Sq, Sk, D = 2, 4, 2, 64, 80, 128
+    dt = torch.float16
+    q = torch.zeros(B, Hq, Sq, D, dtype=dt); k = torch.zeros(B, Hk, Sk, D, dtype=dt); v = torch.zeros_like(k)
+    o = torch.zeros_like(q); do = torch.zeros_like(q); dq = torch.zeros_like(q)
+    dk = torch.zeros_like(k); dv = torch.zeros_like(v)
+    L = torch.zeros(B * Hq, Sq); delta = torch.zeros_like(L)
+    null = torch.empty(0, dtype=torch.uint64)
+    p = attn_bwd_params()
+    flash._fill_bwd(p, q, k, v, None, 0.1, o, do, dq, dk, dv, None, None, L, delta, 0.0, null, null, 0, True)
+    assert validate_bwd(p, attn_bwd_params.kVersion) == E.hipSuccess
+    assert validate_bwd(p, 5) == E.hipErrorInvalidSymbol
+    opt = attn_options(); opt.force_backend_index = 2                          # assembly backend of the reference
+    assert validate_bwd(p, 6, opt) == E.hipErrorPeerAccessUnsupported
+    opt.force_backend_index = 1
+    assert validate_bwd(p, 6, opt) == E.hipSuccess
+    p.D = None                                                                 # no delta: split cannot run
+    opt.force_backend_index = 0
+    assert validate_bwd(p, 6, opt) == E.hipErrorInvalidValue
+    assert validate_bwd(p, 6) == E.hipSuccess                                  # library falls to fused
+
+
+def test_tile_intervals_against_brute_force_and_reference_algebra():
+    L = _lib()
+    rnd = random.Random(99)
+    out = (ctypes.c_int32 * 6)()
+    for _ in range(3000):
+        BM = rnd.choice([16, 32, 64]); BN = rnd.choice([16, 32, 64])
+        sq = rnd.randint(1, 160); sk = rnd.randint(1, 160)
+        causal = rnd.random() < 0.8
+        if rnd.random() < 0.3:
+            wl = wr = rnd.choice([iv.TOP_LEFT, iv.BOTTOM_RIGHT])
+        else:
+            wl = rnd.randint(-30, 180); wr = rnd.randint(-30, 180)
+        start = BM * rnd.randint(0, (sq - 1) // BM)
+        ct = 3 if causal else 0
+        assert L.lib.fa_tile_intervals(ct, wl, wr, start, sq, sk, BM, BN, out) == 0
+        lb, fb, rb = [set(range(out[i], out[i + 1] + 1)) if out[i] <= out[i + 1] else set() for i in (0, 2, 4)]
+        pwl, pwr = iv.parse_window(ct, wl, wr, sq, sk) if causal else (0, 0)
+        rows = range(start, min(start + BM, sq))
+        nblk = (sk + BN - 1) // BN
+        assert not (lb & fb) and not (lb & rb) and not (fb & rb)
+        assert all(0 <= b < nblk for b in lb | fb | rb)
+        for b in range(nblk):
+            vis = [iv.visible(m, n, sq, sk, causal, pwl, pwr) for m in rows for n in range(b * BN, b * BN + BN)]
+            if any(vis):
+                assert b in (lb | fb | rb)
+            if b in fb:
+                assert all(vis)
+        # the reference's algebra (oracle restatement) never calls a block "full" that we must mask
+        # when the tile is not ragged in q, and its union covers ours
+        r = iv.calculate_intervals(causal, pwl, pwr, start, sq, sk, start + BM > sq, BM, BN)
+        ref_full = set(range(r[2], r[3] + 1)) if r[2] <= r[3] else set()
+        ref_all = ref_full | (set(range(r[0], r[1] + 1)) if r[0] <= r[1] else set()) \
+            | (set(range(r[4], r[5] + 1)) if r[4] <= r[5] else set())
+        assert ref_full <= fb
+        assert {b for b in (lb | fb | rb)} <= {b for b in ref_all} | fb
