@@ -1,0 +1,193 @@
+"""GPU parity tests for the packed-sequence (compact varlen) path, the dropout
+mask (bit-exact against the Philox closed form), the reference's known-answer
+tests, and size-independent properties at the BASELINE sizes."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from _util import FUDGE, LSE_ATOL, check, make_inputs
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _u64(x):
+    return torch.tensor([x], dtype=torch.int64, device=DEV).view(torch.uint64)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('D', [64, 128])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_compact_varlen_gqa(dtype, D, causal, backend):
+    # seqlens drawn as the reference does (tests/test_varlen.py:34-47)
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
+    from oracle import fa_ref
+    np.random.seed(8139)
+    lens = np.random.choice([4, 8, 63, 64, 128, 143, 301], size=6)
+    T = int(lens.sum())
+    Hq, Hk = 8, 2
+    cu = [0] + np.cumsum(lens).tolist()
+    g = torch.Generator().manual_seed(5)
+    # THD storage viewed as (1, H, T, D) (tests/_common_test.py:677-678)
+    mk = lambda H: torch.randn(1, T, H, D, generator=g).to(dtype).to(DEV).transpose(1, 2)
+    q, k, v, do = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+    sm = 1.0 / math.sqrt(D)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend)
+    o, _, L = attention_varlen(qg, kg, vg, lens, lens, causal, sm, 0.0, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    assert L.shape == (Hq, T)
+    ct, wl, wr = flash.translate_causal(causal)
+    f = lambda t: t.float()
+    ro, rl = fa_ref.varlen_fwd_ref(f(q), f(k), f(v), cu, cu, sm, ct, wl, wr)
+    lo, ll = fa_ref.varlen_fwd_ref(q, k, v, cu, cu, sm, ct, wl, wr)
+    check('out', o, ro, lo, FUDGE['out'])
+    assert (L - rl).abs().max().item() <= LSE_ATOL
+    rg = fa_ref.varlen_bwd_ref(f(q), f(k), f(v), cu, cu, sm, ro, f(do), rl, ct, wl, wr)
+    lg = fa_ref.varlen_bwd_ref(q, k, v, cu, cu, sm, lo, do, ll.to(dtype), ct, wl, wr)
+    check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
+    check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
+    check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
+
+
+def test_varlen_dropout_mask_uses_sequence_index_and_max_seqlens():
+    from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
+    from oracle import fa_ref, philox
+    lens = np.array([37, 128, 5, 90])
+    T = int(lens.sum()); H = 4; D = 64
+    cu = [0] + np.cumsum(lens).tolist()
+    g = torch.Generator().manual_seed(1)
+    mk = lambda: torch.randn(1, H, T, D, generator=g).to(torch.float16).to(DEV)
+    q, k, v = mk(), mk(), mk()
+    ext = AttentionExtraArgs(return_encoded_softmax=True, return_logsumexp=True)
+    p = 0.3
+    o, enc, L = attention_varlen(q, k, v, lens, lens, True, 0.125, p, ext)
+    torch.cuda.synchronize()
+    mq = int(lens.max())
+    keep = philox.dropout_keep_mask(len(lens), H, mq, mq, p, ext.philox_seed, ext.philox_offset1 + ext.philox_offset2)
+    assert np.array_equal((enc >= 0).cpu().numpy(), keep)
+    keeps = [torch.from_numpy(keep[i:i + 1, :, :lens[i], :lens[i]]).to(DEV) for i in range(len(lens))]
+    ro, _ = fa_ref.varlen_fwd_ref(q.float(), k.float(), v.float(), cu, cu, 0.125, 3, -2147483647, -2147483647, p, keeps)
+    lo, _ = fa_ref.varlen_fwd_ref(q, k, v, cu, cu, 0.125, 3, -2147483647, -2147483647, p, keeps)
+    check('out', o, ro, lo, FUDGE['out'])
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('shape', [(2, 3, 70, 131), (1, 2, 64, 32), (1, 1, 1, 5)])
+@pytest.mark.parametrize('p', [0.1, 0.5])
+def test_encoded_softmax_is_bit_exact(dtype, shape, p):
+    from aotriton_amd import flash
+    from oracle import philox
+    B, H, Sq, Sk = shape
+    sk8 = (Sk + 7) // 8 * 8
+    r = torch.zeros(B, H, Sq, sk8, dtype=dtype, device=DEV)[..., :Sk]
+    seed, off1, off2 = 0x1234, (1 << 32) - 3, 9
+    assert flash.debug_simulate_encoded_softmax(r, p, _u64(seed), _u64(off1), off2) == flash.hipError_t.hipSuccess
+    torch.cuda.synchronize()
+    keep = philox.dropout_keep_mask(B, H, Sq, Sk, p, seed, off1 + off2)
+    assert set(torch.unique(r.float()).tolist()) <= {0.5, -0.5}
+    assert np.array_equal((r >= 0).cpu().numpy(), keep)
+
+
+def test_config5_mask_first_words_and_popcount():
+    """BASELINE config 5 mask (seed 0x1234, offset 0, p=0.1, 8192x8192) on sampled
+    (b, h) slices: bit-exact rows against the oracle and a keep-rate check."""
+    from aotriton_amd import flash
+    from oracle import philox
+    S = 8192
+    B, H = 2, 16
+    r = torch.empty(1, 1, S, S, dtype=torch.float16, device=DEV)
+    # the (b, h) slice is selected through the offset: base + (b*H + h) * S * S/4
+    for (b, h) in [(0, 0), (1, 7)]:
+        off = (b * H + h) * S * (S // 4)
+        assert flash.debug_simulate_encoded_softmax(r, 0.1, _u64(0x1234), _u64(0), off) == 0
+        got = (r[0, 0] >= 0)
+        rows = (0, 1, 4095, 8191)
+        for m in rows:
+            exp = philox.dropout_keep_mask(B, H, S, S, 0.1, 0x1234, 0, rows=(m, m + 1), b_sel=[b], h_sel=[h])[0, 0, 0]
+            assert np.array_equal(got[m].cpu().numpy(), exp)
+        rate = got.float().mean().item()
+        assert abs(rate - 0.9) < 2e-4, rate
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_logsumexp_scaling_known_answer(dtype):
+    # modules/flash/tests/_core_test_backward.py:333-351, embedded in a built head dim
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    D = 64
+    e = torch.zeros(1, 1, 16, D, dtype=dtype, device=DEV)
+    e[0, 0, :, :16] = torch.eye(16, dtype=dtype, device=DEV)
+    o, _, L = attention(e, e, e, None, False, 1.0 / math.sqrt(16), 0.0, AttentionExtraArgs(return_logsumexp=True))
+    assert torch.allclose(L, torch.full_like(L, 2.79018449783325195))
+
+
+@pytest.mark.parametrize('D', [64, 128, 256])
+def test_large_bf16_values_do_not_give_nan(D):
+    # modules/flash/tests/_core_test_backward.py:353-374
+    from aotriton_amd.autograd import attention
+    x = torch.full((1, 1, 1, D), 133120.0, dtype=torch.bfloat16, device=DEV)
+    o, _, _ = attention(x, x.clone(), x.clone(), None, False, 0.125, 0.0)
+    assert not torch.isnan(o).any()
+
+
+@pytest.mark.parametrize('causal', [True, (3, 2)])
+def test_sm_scale_zero_with_masks(causal):
+    # -inf * 0 must not become NaN (fwd_kernel_inner.py:207-211)
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    q, k, v, _, do = make_inputs(1, 2, 2, 77, 91, 64, torch.float16, DEV)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    o, _, L = attention(qg, kg, vg, None, causal, 0.0, 0.0, AttentionExtraArgs(return_logsumexp=True))
+    o.backward(do)
+    ct, wl, wr = flash.translate_causal(causal)
+    ro, rl, _ = fa_ref.attn_fwd_ref(q.float(), k.float(), v.float(), None, 0.0, ct, wl, wr)
+    lo, _, _ = fa_ref.attn_fwd_ref(q, k, v, None, 0.0, ct, wl, wr)
+    check('out', o, ro, lo, FUDGE['out'])
+    for t in (qg.grad, kg.grad, vg.grad):
+        assert torch.isfinite(t).all()
+
+
+def test_headline_size_properties():
+    """B4 H32 S4096 D128 bf16 causal: properties that hold at any size.
+    (1) row 0 of every head attends only to key 0: O[0] == V[0], LSE[0] == s00;
+    (2) a sampled head matches the oracle; (3) the backward's dV column sums:
+    sum_n dV[n] == sum_m dO[m] (rows of P sum to one)."""
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    B, H, S, D = 4, 32, 4096, 128
+    g = torch.Generator(device='cpu').manual_seed(1234)
+    mk = lambda: torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(DEV)
+    q, k, v, do = mk(), mk(), mk(), mk()
+    sm = 1.0 / math.sqrt(D)
+    for backend in (0, 1):
+        qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+        o, _, L = attention(qg, kg, vg, None, True, sm, 0.0,
+                            AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend))
+        o.backward(do)
+        torch.cuda.synchronize()
+        assert torch.equal(o[:, :, 0], v[:, :, 0])
+        s00 = (q[:, :, 0].float() * k[:, :, 0].float()).sum(-1) * sm
+        assert torch.allclose(L.view(B, H, S)[:, :, 0], s00, atol=1e-4, rtol=1e-5)
+        assert not torch.isnan(o).any() and not torch.isnan(L).any()
+        for (b, h) in [(0, 0), (3, 31)]:
+            sl = lambda t: t[b:b + 1, h:h + 1]
+            ro, rl, _ = fa_ref.attn_fwd_ref(sl(q).float(), sl(k).float(), sl(v).float(), None, sm, 3, -2147483647, -2147483647)
+            lo, ll, _ = fa_ref.attn_fwd_ref(sl(q), sl(k), sl(v), None, sm, 3, -2147483647, -2147483647)
+            check('out', sl(o), ro, lo, FUDGE['out'])
+            assert (L.view(B, H, S)[b, h] - rl[0, 0]).abs().max().item() <= LSE_ATOL
+            rg = fa_ref.attn_bwd_ref(sl(q).float(), sl(k).float(), sl(v).float(), None, sm, ro, sl(do).float(), rl,
+                                     3, -2147483647, -2147483647)
+            lg = fa_ref.attn_bwd_ref(sl(q), sl(k), sl(v), None, sm, lo, sl(do), ll.to(torch.bfloat16), 3,
+                                     -2147483647, -2147483647)
+            check('dq', sl(qg.grad), rg[0], lg[0], FUDGE['dq'])
+            check('dk', sl(kg.grad), rg[1], lg[1], FUDGE['dk'])
+            check('dv', sl(vg.grad), rg[2], lg[2], FUDGE['dv'])
+        colsum = vg.grad.float().sum(dim=2)
+        dosum = do.float().sum(dim=2)
+        assert (colsum - dosum).abs().max().item() < 0.5, (colsum - dosum).abs().max().item()
