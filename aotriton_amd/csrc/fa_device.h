@@ -30,13 +30,29 @@ using f32x4 = vec<float, 4>;
 constexpr float kLog2e = 1.44269504089f;       // modules/flash/kernel/fwd_kernel.py:422
 constexpr float kLn2 = 0.6931471824645996f;    // modules/flash/kernel/fwd_kernel.py:610-612
 constexpr float kRcpLn2 = 1.4426950408889634f; // modules/flash/kernel/bwd_inner_dk_dv.py:185
-constexpr float kNegBig = -3.40282e+38f;       // modules/flash/kernel/fwd_kernel.py:417
+// Running-max seed.  The reference seeds with -3.40282e38 (fwd_kernel.py:417); a
+// smaller magnitude keeps max*scale finite so that -inf scores never meet -inf maxima.
+constexpr float kNegBig = -1.0e30f;
 
 template <typename T> struct Traits;
+
+// ds_read_b64_tr_b16: 16 lanes x 4 16-bit elements, transposed on the way out of LDS.
+typedef short tr_raw_t __attribute__((__vector_size__(4 * sizeof(short))));
+__device__ __forceinline__ tr_raw_t lds_read_tr_raw(const void* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tr_raw_t*)(p));
+}
 
 template <> struct Traits<bf16_t> {
   using op_t = vec<__bf16, 8>;
   using q4_t = vec<__bf16, 4>;
+  using p2_t = vec<__bf16, 2>;
+  static __device__ __forceinline__ q4_t lds_read_tr(const bf16_t* p) {
+    return __builtin_bit_cast(q4_t, lds_read_tr_raw(p));
+  }
+  static __device__ __forceinline__ float dot2_ones(p2_t a, float acc) {
+    const p2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(a, ones, acc, false);
+  }
   static __device__ __forceinline__ f32x16 mfma(op_t a, op_t b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -46,6 +62,14 @@ template <> struct Traits<bf16_t> {
 template <> struct Traits<f16_t> {
   using op_t = vec<_Float16, 8>;
   using q4_t = vec<_Float16, 4>;
+  using p2_t = vec<_Float16, 2>;
+  static __device__ __forceinline__ q4_t lds_read_tr(const f16_t* p) {
+    return __builtin_bit_cast(q4_t, lds_read_tr_raw(p));
+  }
+  static __device__ __forceinline__ float dot2_ones(p2_t a, float acc) {
+    const p2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(a, ones, acc, false);
+  }
   static __device__ __forceinline__ f32x16 mfma(op_t a, op_t b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -59,6 +83,31 @@ __device__ __forceinline__ typename Traits<T>::op_t pack8(const f32x16& s, int h
 #pragma unroll
   for (int j = 0; j < 8; ++j) r[j] = Traits<T>::cvt(s[8 * half + j]);
   return r;
+}
+
+// MFMA operand whose 8 k-slots are rows (kbase + 8*w + 4*hi + j) of a row-major LDS
+// tile and whose M/N index (lane%32) is the column: two transposing reads.  `p`
+// must already point at row (4*hi + (lane%16)/4), column (16*((lane/16)%2) + 4*(lane%4))
+// of the 32-column block; rstr is the row stride in elements.
+// Within each group of 16 lanes the hardware returns to lane i, slot j, the element
+// (i%4) of the 8 bytes addressed by lane (4*j + i/4).
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::op_t lds_read_tr8(const T* p, int rstr) {
+  const typename Traits<T>::q4_t lo = Traits<T>::lds_read_tr(p);
+  const typename Traits<T>::q4_t hi = Traits<T>::lds_read_tr(p + 8 * rstr);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Sum of the 8 (already rounded) elements of an operand, added to acc.
+template <typename T>
+__device__ __forceinline__ float sum8(typename Traits<T>::op_t v, float acc) {
+  using p2_t = typename Traits<T>::p2_t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const p2_t pr = {v[2 * i], v[2 * i + 1]};
+    acc = Traits<T>::dot2_ones(pr, acc);
+  }
+  return acc;
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

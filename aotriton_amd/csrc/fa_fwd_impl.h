@@ -9,9 +9,10 @@
 // columns of every 32-key block, so row max / row sum are in-lane plus a single
 // cross-half exchange.  Per K/V tile of BN keys:
 //   S^T (keys x queries) = K_tile . Q^T        A = K rows from LDS, B = Q in registers
-//   O^T (d x queries)   += V_tile^T . P^T      A = V^T rows from LDS, B = P from the S^T accumulators
-// K is staged row-major in LDS; V is staged transposed ([d][key], keys permuted
-// by tr_pos) so that both A operands are single 16-byte LDS reads.
+//   O^T (d x queries)   += V_tile^T . P^T      A = V^T from LDS,    B = P from the S^T accumulators
+// Both tiles are staged row-major.  K rows are padded by 16 B (conflict-free
+// 16-byte row reads); V rows are padded by 64 B so that the transposing LDS reads
+// (ds_read_b64_tr_b16: 4 rows x 64 B per half-wave) sweep all banks once.
 #pragma once
 #include <type_traits>
 
@@ -21,10 +22,10 @@ namespace fa {
 
 template <int D, int BN>
 struct FwdSmem {
-  static constexpr int KSTR = D + 8;     // +16 B per row: conflict-free b128 reads
-  static constexpr int VSTR = BN + 8;
+  static constexpr int KSTR = D + 8;     // +16 B per row
+  static constexpr int VSTR = D + 32;    // +64 B per row
   static constexpr int K_ELEMS = BN * KSTR;
-  static constexpr int V_ELEMS = D * VSTR;
+  static constexpr int V_ELEMS = BN * VSTR;
   static constexpr int STAGES = 2;
   static constexpr int BYTES = STAGES * (K_ELEMS + V_ELEMS) * 2;
 };
@@ -44,10 +45,8 @@ void fwd_kernel(const FwdArgs a) {
   constexpr int DB = D / 32;    // 32-wide blocks of the head dim
   constexpr int TS = BN / 16;   // k-steps of O^T += V^T P^T
   constexpr int KSTR = SM::KSTR, VSTR = SM::VSTR;
-  constexpr int K_CH = (BN * D / 8) / NT;                 // 16-byte chunks of K per thread
-  constexpr int V_BLK = (BN / 4) * (D / 8);               // 4-key x 8-d blocks of V
-  constexpr int V_PT = (V_BLK + NT - 1) / NT;
-  static_assert((BN * D / 8) % NT == 0, "K tile must split evenly");
+  constexpr int CH = (BN * D / 8) / NT;                   // 16-byte chunks per thread, per tensor
+  static_assert((BN * D / 8) % NT == 0, "tile must split evenly");
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   T* Ks = reinterpret_cast<T*>(smem_raw);
@@ -123,36 +122,45 @@ void fwd_kernel(const FwdArgs a) {
   if (kDropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
 
   // ---- global -> register -> LDS staging -------------------------------------
-  op_t kreg[K_CH];
-  op_t vreg[V_PT][4];
+  // Thread-constant offsets inside a tile; the tile base is wave-uniform.
+  op_t kreg[CH], vreg[CH];
+  uint32_t koff[CH], voff[CH];
+  int lrow[CH];
+  uint32_t ldsk[CH], ldsv[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int idx = tid + i * NT;
+    const int r = idx / (D / 8), cc = idx % (D / 8);
+    lrow[i] = r;
+    koff[i] = (uint32_t)(r * (int)a.sk.s + cc * 8);
+    voff[i] = (uint32_t)(r * (int)a.sv.s + cc * 8);
+    ldsk[i] = (uint32_t)(r * KSTR + cc * 8);
+    ldsv[i] = (uint32_t)(r * VSTR + cc * 8);
+  }
 
   auto load_tile = [&](int j) {
-    const int n0 = j * BN;
+    const T* kt = kbase + (int64_t)j * BN * a.sk.s;
+    const T* vt = vbase + (int64_t)j * BN * a.sv.s;
+    if ((j + 1) * BN <= si.seqlen_k) {
 #pragma unroll
-    for (int i = 0; i < K_CH; ++i) {
-      const int idx = tid + i * NT;
-      const int r = idx / (D / 8), cc = idx % (D / 8);
-      int n = n0 + r;
-      n = n < si.seqlen_k ? n : si.seqlen_k - 1;
-      kreg[i] = *reinterpret_cast<const op_t*>(kbase + (int64_t)n * a.sk.s + cc * 8);
-    }
+      for (int i = 0; i < CH; ++i) kreg[i] = *reinterpret_cast<const op_t*>(kt + koff[i]);
 #pragma unroll
-    for (int i = 0; i < V_PT; ++i) {
-      const int blk = tid + i * NT;
-      if (V_BLK % NT == 0 || blk < V_BLK) {
-        const int kb = blk / (D / 8), dbk = blk % (D / 8);
+      for (int i = 0; i < CH; ++i) vreg[i] = *reinterpret_cast<const op_t*>(vt + voff[i]);
+    } else {
+      // ragged last tile: rows past the end are clamped (K) / zeroed (V: P is 0 there)
+      const int nvalid = si.seqlen_k - j * BN;
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          int n = n0 + 4 * kb + rr;
-          const bool ok = n < si.seqlen_k;
-          n = ok ? n : si.seqlen_k - 1;
-          op_t x = *reinterpret_cast<const op_t*>(vbase + (int64_t)n * a.sv.s + dbk * 8);
-          if (!ok) {
+      for (int i = 0; i < CH; ++i) {
+        const bool ok = lrow[i] < nvalid;
+        const int cc8 = (tid + i * NT) % (D / 8) * 8;
+        const int r = ok ? lrow[i] : nvalid - 1;
+        kreg[i] = *reinterpret_cast<const op_t*>(kt + (int64_t)r * a.sk.s + cc8);
+        op_t x = *reinterpret_cast<const op_t*>(vt + (int64_t)r * a.sv.s + cc8);
+        if (!ok) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = 0;   // P is 0 there, keep 0*V finite
-          }
-          vreg[i][rr] = x;
+          for (int e = 0; e < 8; ++e) x[e] = 0;
         }
+        vreg[i] = x;
       }
     }
   };
@@ -161,24 +169,9 @@ void fwd_kernel(const FwdArgs a) {
     T* ks = Ks + stage * SM::K_ELEMS;
     T* vs = Vs + stage * SM::V_ELEMS;
 #pragma unroll
-    for (int i = 0; i < K_CH; ++i) {
-      const int idx = tid + i * NT;
-      const int r = idx / (D / 8), cc = idx % (D / 8);
-      *reinterpret_cast<op_t*>(ks + r * KSTR + cc * 8) = kreg[i];
-    }
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<op_t*>(ks + ldsk[i]) = kreg[i];
 #pragma unroll
-    for (int i = 0; i < V_PT; ++i) {
-      const int blk = tid + i * NT;
-      if (V_BLK % NT == 0 || blk < V_BLK) {
-        const int kb = blk / (D / 8), dbk = blk % (D / 8);
-        const int pos = tr_pos(4 * kb);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          q4_t t4 = {vreg[i][0][e], vreg[i][1][e], vreg[i][2][e], vreg[i][3][e]};
-          *reinterpret_cast<q4_t*>(vs + (dbk * 8 + e) * VSTR + pos) = t4;
-        }
-      }
-    }
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<op_t*>(vs + ldsv[i]) = vreg[i];
   };
 
   // ---- online softmax state --------------------------------------------------
@@ -187,13 +180,21 @@ void fwd_kernel(const FwdArgs a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
-  float m_i = kNegBig;   // fwd_kernel.py:417
+  float m_i = kNegBig;   // running max, in the units of `s` below
   float l_i = 0.f;       // per-lane partial row sum (its half of the columns)
   const float qk_scale = a.sm_scale * kLog2e;
+  // Fast path: the max is taken on the raw scores and the scale is folded into the
+  // exponent, exp2(s*c - m*c), which needs c > 0.  With a bias (added after
+  // scaling, fwd_kernel_inner.py:166-187) or c <= 0 the scores are scaled first.
+  const bool prescale = kBias || !(qk_scale > 0.f);
+  const float sc = prescale ? 1.0f : qk_scale;
+
+  // lane-constant part of the V^T operand address (see lds_read_tr8)
+  const int v_lane = (4 * hi + (lane & 15) / 4) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   auto compute = [&](int j, int stage, bool masked) {
     const T* ks = Ks + stage * SM::K_ELEMS + c * KSTR + hi * 8;
-    const T* vs = Vs + stage * SM::V_ELEMS + c * VSTR + hi * 8;
+    const T* vs = Vs + stage * SM::V_ELEMS + v_lane;
     f32x16 s[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -217,14 +218,14 @@ void fwd_kernel(const FwdArgs a) {
     // first V^T operands: in flight while the softmax runs
     op_t va[2][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) va[0][db] = *reinterpret_cast<const op_t*>(vs + db * 32 * VSTR);
+    for (int db = 0; db < DB; ++db) va[0][db] = lds_read_tr8<T>(vs + db * 32, VSTR);
 
-    // scale (+bias) (+mask), row max.  Scaling happens before the max
-    // (fwd_kernel_inner.py:166,197-205).
+    if (prescale) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+      for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[mb][i] *= qk_scale;
+        for (int i = 0; i < 16; ++i) s[mb][i] *= qk_scale;
+    }
     if (kBias) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -253,23 +254,46 @@ void fwd_kernel(const FwdArgs a) {
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
     mx = fmaxf(mx, xor32(mx));
     const float m_new = fmaxf(m_i, mx);
-    const float alpha = fast_exp2(m_i - m_new);
+    const float alpha = fast_exp2((m_i - m_new) * sc);
+    const float msc = m_new * sc;
+    m_i = m_new;
+
+    op_t pb[TS];
     float rs = 0.f;
+    // exp2(s*c - m*c) as one fma is exact enough while |m*c| is small; for huge
+    // scores the rounding of m*c alone would be amplified by exp2, so the
+    // difference is formed first (the trap documented at fwd_kernel_inner.py:197-205).
+    const bool big = __builtin_amdgcn_ballot_w64(!(__builtin_fabsf(msc) < 1024.f)) != 0;
+    if (big) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[mb][i] = fast_exp2((s[mb][i] - m_new) * sc);
+    } else {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[mb][i] = fast_exp2(__builtin_fmaf(s[mb][i], sc, -msc));
+    }
+    // the row sum is over the fp32, undropped p (fwd_kernel_inner.py:213-214)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint32_t keep = 0xF;
-        if (kDropout) keep = dropout_keep4(ds, row, j * BN + mb * 32 + 8 * g + 4 * hi);
+      for (int i = 0; i < 16; ++i) rs += s[mb][i];
+    if (kDropout) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float p = fast_exp2(s[mb][4 * g + r] - m_new);
-          rs += p;                                     // l sums the undropped p (:213-214)
-          s[mb][4 * g + r] = (!kDropout || ((keep >> r) & 1u)) ? p : 0.f;
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint32_t keep = dropout_keep4(ds, row, j * BN + mb * 32 + 8 * g + 4 * hi);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[mb][4 * g + r] = ((keep >> r) & 1u) ? s[mb][4 * g + r] : 0.f;
         }
-      }
+    }
+    // P is cast to V's dtype for the second GEMM (:274)
+#pragma unroll
+    for (int t = 0; t < TS; ++t) pb[t] = pack8<T>(s[t / 2], t % 2);
     l_i = l_i * alpha + rs;
-    m_i = m_new;
     // rescale the accumulator only when some row of this wave moved its max
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
@@ -277,17 +301,13 @@ void fwd_kernel(const FwdArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
     }
-
-    op_t pb[TS];
-#pragma unroll
-    for (int t = 0; t < TS; ++t) pb[t] = pack8<T>(s[t / 2], t % 2);   // P cast to V's dtype (:274)
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       if (t + 1 < TS) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          va[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(vs + db * 32 * VSTR + (t + 1) * 16);
+          va[(t + 1) & 1][db] = lds_read_tr8<T>(vs + (t + 1) * 16 * VSTR + db * 32, VSTR);
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) o[db] = Tr::mfma(va[t & 1][db], pb[t], o[db]);
@@ -323,11 +343,11 @@ void fwd_kernel(const FwdArgs a) {
         *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
       }
     if (lse_ptr && hi == 0)
-      lse_ptr[row] = alive ? (m_i + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
+      lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
   }
 }
 
-// Tile table: one entry per (dtype size is irrelevant here) head dim.
+// Tile table: one entry per head dim.
 template <int D> struct FwdTile;
 template <> struct FwdTile<64>  { static constexpr int NW = 4, BN = 64; };
 template <> struct FwdTile<128> { static constexpr int NW = 4, BN = 64; };
