@@ -253,7 +253,13 @@ void fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
     mx = fmaxf(mx, xor32(mx));
-    const float m_new = fmaxf(m_i, mx);
+    // Lazy rescaling: a row adopts the new maximum only when it grew by more than
+    // 2^8 in the exponent domain; until then p may exceed 1 (at most 256), which
+    // fp32 accumulation and the 16-bit P operand absorb, and the final O = acc / l
+    // is unchanged because l is accumulated against the same reference.
+    const float m_cand = fmaxf(m_i, mx);
+    const bool upd = (m_cand - m_i) * sc > 8.0f;
+    const float m_new = upd ? m_cand : m_i;
     const float alpha = fast_exp2((m_i - m_new) * sc);
     const float msc = m_new * sc;
     m_i = m_new;
@@ -295,7 +301,7 @@ void fwd_kernel(const FwdArgs a) {
     for (int t = 0; t < TS; ++t) pb[t] = pack8<T>(s[t / 2], t % 2);
     l_i = l_i * alpha + rs;
     // rescale the accumulator only when some row of this wave moved its max
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+    if (__builtin_amdgcn_ballot_w64(upd) != 0) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
