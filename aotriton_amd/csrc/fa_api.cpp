@@ -323,9 +323,16 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   const fa::TileShape t = fa::fwd_tile_shape(s.d);
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
-  out->grid[0] = s.hq;
-  out->grid[1] = (s.max_sq + t.block_m - 1) / t.block_m;
-  out->grid[2] = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+  {
+    const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+    const int zh_per_xcd = (nz * s.hq + fa::kNumXcd - 1) / fa::kNumXcd;
+    const int ratio = s.hq / s.hk;
+    const int zg = ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2;
+    const int groups = (zh_per_xcd + zg - 1) / zg;
+    out->grid[0] = fa::kNumXcd * groups * zg * ((s.max_sq + t.block_m - 1) / t.block_m);
+    out->grid[1] = 1;
+    out->grid[2] = 1;
+  }
   out->backend_index = 0;
   out->head_dim = s.d;
   out->flags = (s.windowed ? 1 : 0) | (s.bias ? 2 : 0) | (s.dropout ? 4 : 0) | (s.num_seqlens != 0 ? 8 : 0);

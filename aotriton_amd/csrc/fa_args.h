@@ -5,6 +5,8 @@
 
 namespace fa {
 
+constexpr int kNumXcd = 8;   // MI355X: 8 XCDs x 32 CUs, one L2 each
+
 struct Strides3 {   // batch, head, row
   int64_t z, h, s;
 };
@@ -45,6 +47,9 @@ struct FwdArgs {
   uint64_t* seed_out; uint64_t* offset_out;
   int32_t* atomic_counter;
   int32_t num_m_tiles;
+  int32_t num_zh;        // (batch or sequences) x q-heads
+  int32_t zh_per_xcd;    // ceil(num_zh / 8)
+  int32_t zh_group;      // heads walked together on one XCD
 };
 
 struct BwdArgs {

@@ -110,6 +110,21 @@ __device__ __forceinline__ float sum8(typename Traits<T>::op_t v, float acc) {
   return acc;
 }
 
+// acc *= f for an MFMA accumulator that should stay in the accumulator register
+// file: the values are moved out, scaled and moved back explicitly so that the
+// compiler never needs a vector-ALU home for the whole block.
+__device__ __forceinline__ void scale_acc(f32x16& acc, float f) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float t;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[i]));
+    t *= f;
+    float r;
+    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(r) : "v"(t));
+    acc[i] = r;
+  }
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

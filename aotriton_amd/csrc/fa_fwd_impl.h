@@ -55,11 +55,23 @@ void fwd_kernel(const FwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
 
-  const int h = xcd_remap_head(blockIdx.x, a.hq);
-  const int mt = a.num_m_tiles - 1 - (int)blockIdx.y;   // heaviest causal tiles first
-  const int z = blockIdx.z;
+  // 1-D grid.  Consecutive workgroup ids round-robin over the 8 XCDs; each XCD walks
+  // its own contiguous range of (batch, head) pairs in small groups: inside a group
+  // the Q tiles go heaviest-first (causal) with the heads of the group interleaved.
+  // Few heads are in flight per XCD, so their K/V stay in that XCD's L2, and the
+  // stream of groups keeps the CUs of the XCD evenly loaded.
+  const int xcd = blockIdx.x % kNumXcd;
+  const int li = blockIdx.x / kNumXcd;
+  const int per_group = a.zh_group * a.num_m_tiles;
+  const int gi = li / per_group, gr = li % per_group;
+  const int zh_local = gi * a.zh_group + gr % a.zh_group;
+  const int zh = xcd * a.zh_per_xcd + zh_local;
+  if (zh_local >= a.zh_per_xcd || zh >= a.num_zh) return;
+  const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
+  const int z = zh / a.hq;
+  const int h = zh % a.hq;
 
-  if (kDropout && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0) {
+  if (kDropout && blockIdx.x == 0 && tid == 0) {
     // modules/flash/kernel/fwd_kernel.py:199-207
     const uint64_t seed = *a.drop.seed_ptr;
     uint64_t base = a.drop.offset2;
@@ -191,6 +203,16 @@ void fwd_kernel(const FwdArgs a) {
 
   // lane-constant part of the V^T operand address (see lds_read_tr8)
   const int v_lane = (4 * hi + (lane & 15) / 4) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  // last K tile this wave needs: on the causal diagonal the upper waves of a tile
+  // see nothing in the trailing K tiles and only take part in staging and barriers
+  int wave_hi = br.hi;
+  if (kWindowed) {
+    const int64_t wl = (int64_t)(q0 + wave * 32 + 31 < si.seqlen_q ? q0 + wave * 32 + 31 : si.seqlen_q - 1);
+    int64_t cmax = wl + w.right;
+    if (cmax > si.seqlen_k - 1) cmax = si.seqlen_k - 1;
+    wave_hi = cmax < 0 ? -1 : (int)(cmax / BN);
+  }
 
   auto compute = [&](int j, int stage, bool masked) {
     const T* ks = Ks + stage * SM::K_ELEMS + c * KSTR + hi * 8;
@@ -328,7 +350,7 @@ void fwd_kernel(const FwdArgs a) {
   for (int j = br.lo; j <= br.hi; ++j) {
     const int stage = (j - br.lo) & 1;
     if (j < br.hi) load_tile(j + 1);
-    compute(j, stage, !br.is_full(j));
+    if (j <= wave_hi) compute(j, stage, !br.is_full(j));
     if (j < br.hi) store_tile(stage ^ 1);
     __syncthreads();
   }
@@ -355,8 +377,8 @@ void fwd_kernel(const FwdArgs a) {
 
 // Tile table: one entry per head dim.
 template <int D> struct FwdTile;
-template <> struct FwdTile<64>  { static constexpr int NW = 4, BN = 64; };
-template <> struct FwdTile<128> { static constexpr int NW = 4, BN = 64; };
+template <> struct FwdTile<64>  { static constexpr int NW = 8, BN = 64; };
+template <> struct FwdTile<128> { static constexpr int NW = 8, BN = 64; };
 template <> struct FwdTile<256> { static constexpr int NW = 4, BN = 32; };
 
 template <typename T, int D, bool kWindowed, bool kBias, bool kDropout>
@@ -380,7 +402,11 @@ hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, 
                                           : a.batch;
   FwdArgs b = a;
   b.num_m_tiles = (a.seq.max_seqlen_q + BM - 1) / BM;
-  dim3 grid(a.hq, b.num_m_tiles, nseq);
+  b.num_zh = nseq * a.hq;
+  b.zh_per_xcd = (b.num_zh + kNumXcd - 1) / kNumXcd;
+  b.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
+  const int groups = (b.zh_per_xcd + b.zh_group - 1) / b.zh_group;
+  dim3 grid((unsigned)(kNumXcd * groups * b.zh_group * b.num_m_tiles));
   const int key = (windowed ? 4 : 0) | (bias ? 2 : 0) | (dropout ? 1 : 0);
   switch (key) {
     case 0: return launch_fwd_variant<T, D, false, false, false>(b, grid, stream);

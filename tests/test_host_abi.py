@@ -122,8 +122,8 @@ def test_validate_fwd_error_contract():
     assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # alibi
     p, keep = _fwd_params()
     err, cfg = query_fwd_config(p)
-    assert err == E.hipSuccess and cfg.block_m == 128 and cfg.head_dim == 128
-    assert list(cfg.grid) == [4, 1, 2]
+    assert err == E.hipSuccess and cfg.block_m == 256 and cfg.head_dim == 128
+    assert list(cfg.grid) == [16, 1, 1]     # 8 XCDs x one group of 2 head slots x 1 Q tile
 
 
 def test_validate_bwd_error_contract():
