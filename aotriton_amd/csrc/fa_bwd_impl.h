@@ -56,23 +56,29 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
 // ---------------------------------------------------------------------------
 // Shared-memory plans
 // ---------------------------------------------------------------------------
+// Every staged tile is row-major.  A tile that is read as rows (16-byte reads, the
+// contraction runs over the head dim) gets rows padded by 16 B; a tile that is read
+// through the transposing LDS loads (the contraction runs over its rows) gets rows
+// padded by 64 B.  Q and dO (dK/dV item) and K (dQ item) are needed both ways and
+// are simply stored twice, once per padding: no register transposes, no bank
+// conflicts on either access pattern.
 template <int D, int BM>
-struct DkDvSmem {   // per stage: Q, dO row-major; Q^T, dO^T transposed; L, delta
+struct DkDvSmem {   // per stage: Q, dO for row reads; Q, dO for transposing reads; L, delta
   static constexpr int RSTR = D + 8;
-  static constexpr int TSTR = BM + 8;
+  static constexpr int TSTR = D + 32;
   static constexpr int ROW_ELEMS = BM * RSTR;
-  static constexpr int TR_ELEMS = D * TSTR;
+  static constexpr int TR_ELEMS = BM * TSTR;
   static constexpr int STAGE_BYTES = (2 * ROW_ELEMS + 2 * TR_ELEMS) * 2 + 2 * BM * 4;
   static constexpr int STAGES = 2;
   static constexpr int BYTES = STAGES * STAGE_BYTES;
 };
 
 template <int D, int BN>
-struct DqSmem {     // per stage: K row-major, K^T transposed, V row-major
+struct DqSmem {     // per stage: K, V for row reads; K for transposing reads
   static constexpr int RSTR = D + 8;
-  static constexpr int TSTR = BN + 8;
+  static constexpr int TSTR = D + 32;
   static constexpr int ROW_ELEMS = BN * RSTR;
-  static constexpr int TR_ELEMS = D * TSTR;
+  static constexpr int TR_ELEMS = BN * TSTR;
   static constexpr int STAGE_BYTES = (2 * ROW_ELEMS + TR_ELEMS) * 2;
   static constexpr int STAGES = 2;
   static constexpr int BYTES = STAGES * STAGE_BYTES;
@@ -82,40 +88,6 @@ template <int D> struct BwdTile;   // NW waves; dK/dV: BN = 32*NW keys x BM quer
 template <> struct BwdTile<64>  { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
 template <> struct BwdTile<128> { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
 template <> struct BwdTile<256> { static constexpr int NW = 4, DKDV_BM = 32, DQ_BN = 32; };
-
-// A 4-row x 8-column block of a row-major global tile, staged by one thread:
-// written to LDS both row-major (4 x 16 B) and transposed (8 x 8 B).
-template <typename T>
-struct Block4x8 {
-  using op_t = typename Traits<T>::op_t;
-  using q4_t = typename Traits<T>::q4_t;
-  op_t r[4];
-  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int row0, int col0, int nrows) {
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-      const int m = row0 + rr;
-      const bool ok = m < nrows;
-      op_t x = *reinterpret_cast<const op_t*>(base + (int64_t)(ok ? m : nrows - 1) * row_stride + col0);
-      if (!ok) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = 0;
-      }
-      r[rr] = x;
-    }
-  }
-  __device__ __forceinline__ void store_rows(T* dst, int rstr, int lrow0, int col0) const {
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) *reinterpret_cast<op_t*>(dst + (lrow0 + rr) * rstr + col0) = r[rr];
-  }
-  __device__ __forceinline__ void store_transposed(T* dst, int tstr, int lrow0, int col0) const {
-    const int pos = tr_pos(lrow0);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      q4_t t4 = {r[0][e], r[1][e], r[2][e], r[3][e]};
-      *reinterpret_cast<q4_t*>(dst + (col0 + e) * tstr + pos) = t4;
-    }
-  }
-};
 
 // ---------------------------------------------------------------------------
 // dK / dV work item
@@ -131,8 +103,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   constexpr int BN = NW * 32;
   constexpr int KS = D / 16, MB = BM / 32, DB = D / 32, TS = BM / 16;
   constexpr int RSTR = SM::RSTR, TSTR = SM::TSTR;
-  constexpr int NBLK = (BM / 4) * (D / 8);
-  constexpr int BPT = (NBLK + NT - 1) / NT;     // 4x8 blocks per thread, per tensor
+  constexpr int NCH = BM * D / 8;                // 16-byte chunks per tile, per tensor
+  constexpr int CH = (NCH + NT - 1) / NT;        // chunks per thread, per tensor
+  constexpr int LPR = D / 8;                     // lanes that share one row
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
@@ -194,42 +167,69 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   const int ntq = br.hi - br.lo + 1;
   const int total = group * ntq;
   const float qk_scale = a.sm_scale * kLog2e;
+  // lane-constant part of the transposing-read address (see lds_read_tr8)
+  const int tr_lane = (4 * hi + (lane & 15) / 4) * TSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   auto stage_ptr = [&](int stage) { return smem_raw + stage * SM::STAGE_BYTES; };
 
   // ---- staging -----------------------------------------------------------------
-  Block4x8<T> qblk[BPT], doblk[BPT];
+  op_t qch[CH], doch[CH];
   float l_stage = 0.f, d_stage = 0.f;
-  float dpart[BPT][4];
+  float dpart[CH];
+  int crow[CH];
+  uint32_t qoff[CH], dooff[CH], ooff[CH], lrow_off[CH], ltr_off[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int idx = tid + i * NT;
+    const int r = idx / LPR, cc = idx % LPR;
+    crow[i] = r;
+    qoff[i] = (uint32_t)(r * (int)a.sq.s + cc * 8);
+    dooff[i] = (uint32_t)(r * (int)a.sdo.s + cc * 8);
+    ooff[i] = (uint32_t)(r * (int)a.so.s + cc * 8);
+    lrow_off[i] = (uint32_t)(r * RSTR + cc * 8);
+    ltr_off[i] = (uint32_t)(r * TSTR + cc * 8);
+  }
 
   auto load_tile = [&](int it) {
     const int hq = hk * group + it / ntq;
     const int m0 = (br.lo + it % ntq) * BM;
     const T* qb = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)hq * a.sq.h +
-                  (int64_t)si.q_start * a.sq.s;
+                  (int64_t)(si.q_start + m0) * a.sq.s;
     const T* dob = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
-                   (int64_t)hq * a.sdo.h + (int64_t)si.q_start * a.sdo.s;
+                   (int64_t)hq * a.sdo.h + (int64_t)(si.q_start + m0) * a.sdo.s;
+    const T* ob = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z +
+                  (int64_t)hq * a.so.h + (int64_t)(si.q_start + m0) * a.so.s;
+    const int nvalid = si.seqlen_q - m0;          // > 0
+    const bool full = nvalid >= BM;
 #pragma unroll
-    for (int b = 0; b < BPT; ++b) {
-      const int blk = tid + b * NT;
-      if (NBLK % NT == 0 || blk < NBLK) {
-        const int kb = blk / (D / 8), cb = blk % (D / 8);
-        qblk[b].load(qb, a.sq.s, m0 + 4 * kb, cb * 8, si.seqlen_q);
-        doblk[b].load(dob, a.sdo.s, m0 + 4 * kb, cb * 8, si.seqlen_q);
-        if (kInlineDelta) {
-          // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310)
-          const T* ob = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z +
-                        (int64_t)hq * a.so.h + (int64_t)si.q_start * a.so.s;
-          Block4x8<T> oblk;
-          oblk.load(ob, a.so.s, m0 + 4 * kb, cb * 8, si.seqlen_q);
+    for (int i = 0; i < CH; ++i) {
+      if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
+      op_t qv, dv_, ov;
+      if (full) {
+        qv = *reinterpret_cast<const op_t*>(qb + qoff[i]);
+        dv_ = *reinterpret_cast<const op_t*>(dob + dooff[i]);
+        if (kInlineDelta) ov = *reinterpret_cast<const op_t*>(ob + ooff[i]);
+      } else {
+        // ragged last Q tile: rows past the end are zero (they are also masked)
+        const bool ok = crow[i] < nvalid;
+        const int r = ok ? crow[i] : nvalid - 1;
+        const int cc8 = (tid + i * NT) % LPR * 8;
+        qv = *reinterpret_cast<const op_t*>(qb + (int64_t)r * a.sq.s + cc8);
+        dv_ = *reinterpret_cast<const op_t*>(dob + (int64_t)r * a.sdo.s + cc8);
+        if (kInlineDelta) ov = *reinterpret_cast<const op_t*>(ob + (int64_t)r * a.so.s + cc8);
+        if (!ok) {
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            float acc = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc += (float)oblk.r[rr][e] * (float)doblk[b].r[rr][e];
-            dpart[b][rr] = acc;
-          }
+          for (int e = 0; e < 8; ++e) { qv[e] = 0; dv_[e] = 0; }
         }
+      }
+      qch[i] = qv;
+      doch[i] = dv_;
+      if (kInlineDelta) {
+        // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310)
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv_[e];
+        dpart[i] = acc;
       }
     }
     if (tid < BM) {
@@ -250,24 +250,18 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     float* Ls = reinterpret_cast<float*>(dOt + SM::TR_ELEMS);
     float* Ds = Ls + BM;
 #pragma unroll
-    for (int b = 0; b < BPT; ++b) {
-      const int blk = tid + b * NT;
-      if (NBLK % NT == 0 || blk < NBLK) {
-        const int kb = blk / (D / 8), cb = blk % (D / 8);
-        qblk[b].store_rows(Qs, RSTR, 4 * kb, cb * 8);
-        qblk[b].store_transposed(Qt, TSTR, 4 * kb, cb * 8);
-        doblk[b].store_rows(dOs, RSTR, 4 * kb, cb * 8);
-        doblk[b].store_transposed(dOt, TSTR, 4 * kb, cb * 8);
-        if (kInlineDelta) {
-          // the D/8 threads that share a row are consecutive lanes
+    for (int i = 0; i < CH; ++i) {
+      if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
+      *reinterpret_cast<op_t*>(Qs + lrow_off[i]) = qch[i];
+      *reinterpret_cast<op_t*>(Qt + ltr_off[i]) = qch[i];
+      *reinterpret_cast<op_t*>(dOs + lrow_off[i]) = doch[i];
+      *reinterpret_cast<op_t*>(dOt + ltr_off[i]) = doch[i];
+      if (kInlineDelta) {
+        // the LPR threads that share a row are consecutive lanes
+        float acc = dpart[i];
 #pragma unroll
-          for (int rr = 0; rr < 4; ++rr) {
-            float acc = dpart[b][rr];
-#pragma unroll
-            for (int off = (D / 8) / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-            if (cb == 0) Ds[4 * kb + rr] = acc;
-          }
-        }
+        for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if ((tid + i * NT) % LPR == 0) Ds[crow[i]] = acc;
       }
     }
     if (tid < BM) {
@@ -283,7 +277,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     char* sp = stage_ptr(stage);
     const T* Qs = reinterpret_cast<const T*>(sp) + c * RSTR + hi * 8;
     const T* dOs = reinterpret_cast<const T*>(sp) + SM::ROW_ELEMS + c * RSTR + hi * 8;
-    const T* Qt = reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + c * TSTR + hi * 8;
+    const T* Qt = reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + tr_lane;
     const T* dOt = Qt + SM::TR_ELEMS;
     const float* Ls = reinterpret_cast<const float*>(reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + 2 * SM::TR_ELEMS);
     const float* Ds = Ls + BM;
@@ -324,7 +318,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     // first transposed operands in flight during the elementwise part
     op_t ta[2][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = *reinterpret_cast<const op_t*>(dOt + db * 32 * TSTR);
+    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(dOt + db * 32, TSTR);
 
     DropoutState dst{};
     if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
@@ -344,17 +338,20 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         for (int r = 0; r < 4; ++r) {
           const int i = 4 * g + r;
           const int m = m0 + mloc + r;
-          float x = s[mb][i] * qk_scale;
+          // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
+          float x;
           if (kBias) {
             const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
-            x += (float)bptr[(int64_t)mm * a.sb_m] * kLog2e;
+            x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)mm * a.sb_m] * kLog2e) - l4[r];
+          } else {
+            x = __builtin_fmaf(s[mb][i], qk_scale, -l4[r]);
           }
           if (masked) {
             bool vis = (m < si.seqlen_q) & key_ok;
             if (kWindowed) vis = vis & (key <= m + w.right) & (key >= m - w.left);
             x = vis ? x : -__builtin_inff();
           }
-          const float p = fast_exp2(x - l4[r]);          // bwd_inner_dk_dv.py:187-188
+          const float p = fast_exp2(x);
           float pd = p, dpv = dp[mb][i];
           if (kDropout) {
             const bool keep = dropout_keep1(dst, m, key);
@@ -378,20 +375,20 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       if (t + 1 < TS) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(dOt + db * 32 * TSTR + (t + 1) * 16);
+          ta[(t + 1) & 1][db] = lds_read_tr8<T>(dOt + (t + 1) * 16 * TSTR + db * 32, TSTR);
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) dv[db] = Tr::mfma(ta[t & 1][db], pb[t], dv[db]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = *reinterpret_cast<const op_t*>(Qt + db * 32 * TSTR);
+    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Qt + db * 32, TSTR);
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       if (t + 1 < TS) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(Qt + db * 32 * TSTR + (t + 1) * 16);
+          ta[(t + 1) & 1][db] = lds_read_tr8<T>(Qt + (t + 1) * 16 * TSTR + db * 32, TSTR);
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
@@ -441,10 +438,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   constexpr int BM = NW * 32;
   constexpr int KS = D / 16, MB = BN / 32, DB = D / 32, TS = BN / 16;
   constexpr int RSTR = SM::RSTR, TSTR = SM::TSTR;
-  constexpr int NBLK = (BN / 4) * (D / 8);
-  constexpr int BPT = (NBLK + NT - 1) / NT;
-  constexpr int V_CH = (BN * D / 8) / NT;
-  static_assert((BN * D / 8) % NT == 0, "V tile must split evenly");
+  constexpr int CH = (BN * D / 8) / NT;          // 16-byte chunks per thread, per tensor
+  static_assert((BN * D / 8) % NT == 0, "tile must split evenly");
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
@@ -541,26 +536,46 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     for (int i = 0; i < 16; ++i) dq[db][i] = 0.f;
   const float qk_scale = a.sm_scale * kLog2e;
 
-  Block4x8<T> kblk[BPT];
-  op_t vch[V_CH];
+  op_t kch[CH], vch[CH];
+  int crow[CH];
+  uint32_t koff[CH], voff[CH], lrow_off[CH], ltr_off[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int idx = tid + i * NT;
+    const int r = idx / (D / 8), cc = idx % (D / 8);
+    crow[i] = r;
+    koff[i] = (uint32_t)(r * (int)a.sk.s + cc * 8);
+    voff[i] = (uint32_t)(r * (int)a.sv.s + cc * 8);
+    lrow_off[i] = (uint32_t)(r * RSTR + cc * 8);
+    ltr_off[i] = (uint32_t)(r * TSTR + cc * 8);
+  }
+  // lane-constant part of the transposing-read address (see lds_read_tr8)
+  const int tr_lane = (4 * hi + (lane & 15) / 4) * TSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   auto load_tile = [&](int j) {
-    const int nn0 = j * BN;
+    const T* kt = kbase + (int64_t)j * BN * a.sk.s;
+    const T* vt = vbase + (int64_t)j * BN * a.sv.s;
+    if ((j + 1) * BN <= si.seqlen_k) {
 #pragma unroll
-    for (int b = 0; b < BPT; ++b) {
-      const int blk = tid + b * NT;
-      if (NBLK % NT == 0 || blk < NBLK) {
-        const int kb = blk / (D / 8), cb = blk % (D / 8);
-        kblk[b].load(kbase, a.sk.s, nn0 + 4 * kb, cb * 8, si.seqlen_k);
+      for (int i = 0; i < CH; ++i) kch[i] = *reinterpret_cast<const op_t*>(kt + koff[i]);
+#pragma unroll
+      for (int i = 0; i < CH; ++i) vch[i] = *reinterpret_cast<const op_t*>(vt + voff[i]);
+    } else {
+      // ragged last K tile: rows past the end are zero (K: dS is 0 there) / clamped (V)
+      const int nvalid = si.seqlen_k - j * BN;
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        const bool ok = crow[i] < nvalid;
+        const int r = ok ? crow[i] : nvalid - 1;
+        const int cc8 = (tid + i * NT) % (D / 8) * 8;
+        op_t x = *reinterpret_cast<const op_t*>(kt + (int64_t)r * a.sk.s + cc8);
+        if (!ok) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = 0;
+        }
+        kch[i] = x;
+        vch[i] = *reinterpret_cast<const op_t*>(vt + (int64_t)r * a.sv.s + cc8);
       }
-    }
-#pragma unroll
-    for (int i = 0; i < V_CH; ++i) {
-      const int idx = tid + i * NT;
-      const int r = idx / (D / 8), cc = idx % (D / 8);
-      int n = nn0 + r;
-      n = n < si.seqlen_k ? n : si.seqlen_k - 1;
-      vch[i] = *reinterpret_cast<const op_t*>(vbase + (int64_t)n * a.sv.s + cc * 8);
     }
   };
   auto store_tile = [&](int stage) {
@@ -568,27 +583,17 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     T* Vs = Ks + SM::ROW_ELEMS;
     T* Kt = Vs + SM::ROW_ELEMS;
 #pragma unroll
-    for (int b = 0; b < BPT; ++b) {
-      const int blk = tid + b * NT;
-      if (NBLK % NT == 0 || blk < NBLK) {
-        const int kb = blk / (D / 8), cb = blk % (D / 8);
-        kblk[b].store_rows(Ks, RSTR, 4 * kb, cb * 8);
-        kblk[b].store_transposed(Kt, TSTR, 4 * kb, cb * 8);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < V_CH; ++i) {
-      const int idx = tid + i * NT;
-      const int r = idx / (D / 8), cc = idx % (D / 8);
-      *reinterpret_cast<op_t*>(Vs + r * RSTR + cc * 8) = vch[i];
+    for (int i = 0; i < CH; ++i) {
+      *reinterpret_cast<op_t*>(Ks + lrow_off[i]) = kch[i];
+      *reinterpret_cast<op_t*>(Kt + ltr_off[i]) = kch[i];
+      *reinterpret_cast<op_t*>(Vs + lrow_off[i]) = vch[i];
     }
   };
 
   auto compute = [&](int j, int stage, bool masked) {
     const T* Ks = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + c * RSTR + hi * 8;
     const T* Vs = Ks + SM::ROW_ELEMS;
-    const T* Kt = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + 2 * SM::ROW_ELEMS +
-                  c * TSTR + hi * 8;
+    const T* Kt = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + 2 * SM::ROW_ELEMS + tr_lane;
     f32x16 s[MB], dp[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -623,7 +628,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     }
     op_t ta[2][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = *reinterpret_cast<const op_t*>(Kt + db * 32 * TSTR);
+    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Kt + db * 32, TSTR);
 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -636,17 +641,19 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         for (int r = 0; r < 4; ++r) {
           const int i = 4 * g + r;
           const int n = nb + r;
-          float x = s[mb][i] * qk_scale;
+          float x;
           if (kBias) {
             const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
-            x += (float)bptr[(int64_t)nn * a.sb_n] * kLog2e;
+            x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)nn * a.sb_n] * kLog2e) - l_row;
+          } else {
+            x = __builtin_fmaf(s[mb][i], qk_scale, -l_row);
           }
           if (masked) {
             bool vis = n < si.seqlen_k;
             if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
             x = vis ? x : -__builtin_inff();
           }
-          const float p = fast_exp2(x - l_row);
+          const float p = fast_exp2(x);
           float dpv = dp[mb][i];
           if (kDropout) dpv = ((keep >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
           const float dsv = p * (dpv - d_row);
@@ -664,7 +671,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       if (t + 1 < TS) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = *reinterpret_cast<const op_t*>(Kt + db * 32 * TSTR + (t + 1) * 16);
+          ta[(t + 1) & 1][db] = lds_read_tr8<T>(Kt + (t + 1) * 16 * TSTR + db * 32, TSTR);
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) dq[db] = Tr::mfma(ta[t & 1][db], sb[t], dq[db]);
