@@ -271,7 +271,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   };
 
   // ---- one (q-head, Q tile) step -----------------------------------------------
-  auto compute = [&](int it, int stage, bool masked) {
+  auto compute = [&](auto masked_tag, int it, int stage) {
+    constexpr bool masked = decltype(masked_tag)::value;
     const int hq = hk * group + it / ntq;
     const int m0 = (br.lo + it % ntq) * BM;
     char* sp = stage_ptr(stage);
@@ -283,10 +284,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const float* Ds = Ls + BM;
 
     f32x16 s[MB], dp[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     op_t xa[2][MB];
 #pragma unroll
@@ -299,7 +297,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
           xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + (k + 1) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], kreg[k], s[mb]);
+      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], kreg[k], k == 0 ? zero16 : s[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -312,7 +310,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
           xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + (k + 1) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], vreg[k], dp[mb]);
+      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], vreg[k], k == 0 ? zero16 : dp[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
     // first transposed operands in flight during the elementwise part
@@ -399,12 +397,23 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   load_tile(0);
   store_tile(0);
   __syncthreads();
-  for (int it = 0; it < total; ++it) {
+  // Per q-head the Q tiles come as [masked | full | masked]; each run has its own
+  // loop so that the loop bodies are straight-line code.
+  const int n_lb = br.fb_lo <= br.fb_hi ? br.fb_lo - br.lo : ntq;
+  const int n_fb = br.fb_lo <= br.fb_hi ? br.fb_hi - br.fb_lo + 1 : 0;
+  int it = 0;
+  auto step = [&](auto masked_tag) {
     const int stage = it & 1;
     if (it + 1 < total) load_tile(it + 1);
-    compute(it, stage, !br.is_full(br.lo + it % ntq));
+    compute(masked_tag, it, stage);
     if (it + 1 < total) store_tile(stage ^ 1);
     __syncthreads();
+    ++it;
+  };
+  for (int g = 0; g < group; ++g) {
+    for (int e = 0; e < n_lb; ++e) step(std::true_type{});
+    for (int e = 0; e < n_fb; ++e) step(std::false_type{});
+    for (int e = n_lb + n_fb; e < ntq; ++e) step(std::true_type{});
   }
 
   if (key_ok) {
@@ -590,15 +599,13 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     }
   };
 
-  auto compute = [&](int j, int stage, bool masked) {
+  auto compute = [&](auto masked_tag, int j, int stage) {
+    constexpr bool masked = decltype(masked_tag)::value;
     const T* Ks = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + c * RSTR + hi * 8;
     const T* Vs = Ks + SM::ROW_ELEMS;
     const T* Kt = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + 2 * SM::ROW_ELEMS + tr_lane;
     f32x16 s[MB], dp[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     op_t xa[2][MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR);
@@ -610,7 +617,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
           xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + (k + 1) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], qreg[k], s[mb]);
+      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], qreg[k], k == 0 ? zero16 : s[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -623,7 +630,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
           xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + (k + 1) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], doreg[k], dp[mb]);
+      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], doreg[k], k == 0 ? zero16 : dp[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
     op_t ta[2][DB];
@@ -682,12 +689,22 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   load_tile(br.lo);
   store_tile(0);
   __syncthreads();
-  for (int j = br.lo; j <= br.hi; ++j) {
-    const int stage = (j - br.lo) & 1;
-    if (j < br.hi) load_tile(j + 1);
-    compute(j, stage, !br.is_full(j));
-    if (j < br.hi) store_tile(stage ^ 1);
-    __syncthreads();
+  // K tiles come as [masked | full | masked]; one straight-line loop per run
+  {
+    int j = br.lo;
+    auto step = [&](auto masked_tag) {
+      const int stage = (j - br.lo) & 1;
+      if (j < br.hi) load_tile(j + 1);
+      compute(masked_tag, j, stage);
+      if (j < br.hi) store_tile(stage ^ 1);
+      __syncthreads();
+      ++j;
+    };
+    const int full_lo = br.fb_lo <= br.fb_hi ? br.fb_lo : br.hi + 1;
+    const int full_hi = br.fb_lo <= br.fb_hi ? br.fb_hi : br.hi;
+    while (j < full_lo) step(std::true_type{});
+    while (j <= full_hi) step(std::false_type{});
+    while (j <= br.hi) step(std::true_type{});
   }
 
   if (row_ok) {
