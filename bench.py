@@ -25,6 +25,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16/fp16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
 
+# HBM bytes per launch at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# runs scaled by a 256 MiB elementwise probe (summaries and commands: profiles/*.txt).
+# Counters cannot be read from inside this process, so the figures are recorded here.
+HBM_BYTES_PER_LAUNCH = {'fwd_kernel': 6.3881e8, 'bwd_dkdv_kernel': 1.2514e9, 'bwd_dq_kernel': 1.0490e9}
+
 
 def cpu_baseline(B, H, S, D, causal, seed):
     """PyTorch math SDPA on the host CPU, fwd + bwd by autograd, on H_s heads of one
@@ -33,7 +38,7 @@ def cpu_baseline(B, H, S, D, causal, seed):
     from oracle import fa_ref
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
-    h_s = 2
+    h_s = 8
     g = torch.Generator().manual_seed(seed)
     q = torch.randn(1, h_s, S, D, generator=g).requires_grad_()
     k = torch.randn(1, h_s, S, D, generator=g).requires_grad_()
@@ -42,7 +47,7 @@ def cpu_baseline(B, H, S, D, causal, seed):
     ct, wl, wr = (3, -2147483647, -2147483647) if causal else (0, 0, 0)
     sm = 1.0 / math.sqrt(D)
     fa_ref.sdpa_math_ref(q, k, v, None, sm, ct, wl, wr).backward(do)   # warm-up
-    reps = 2
+    reps = 4
     t0 = time.perf_counter()
     for _ in range(reps):
         q.grad = k.grad = v.grad = None
@@ -63,6 +68,9 @@ def main():
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu', action='store_true', help='skip the host-CPU baseline leg')
+    ap.add_argument('--traffic-probe', action='store_true',
+                    help='also run one elementwise kernel of known HBM traffic (256 MiB read + 256 MiB '
+                         'written) so that FETCH_SIZE / WRITE_SIZE counters can be scaled')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU only (attention shards by batch/head with no '
@@ -122,6 +130,13 @@ def main():
         e1.synchronize()
         return e0.elapsed_time(e1) / n
 
+    if args.traffic_probe:
+        x = torch.zeros(64 * 1024 * 1024, device=dev, dtype=torch.float32)
+        y = torch.empty_like(x)
+        torch.add(x, 1.0, out=y)          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del x, y
+
     for _ in range(args.warmup):
         fwd()
         bwd(0)
@@ -159,8 +174,8 @@ def main():
     dom = max(kernels, key=lambda kname: kernels[kname][0])
     dom_ms, dom_fl = kernels[dom]
     roofline = {'bound': 'mfma', 'kernel': dom, 'achieved': tf(dom_fl, dom_ms), 'peak': PEAK_BF16_TFLOPS,
-                'unit': 'TFLOP/s', 'frac': tf(dom_fl, dom_ms) / PEAK_BF16_TFLOPS, 'traffic': None,
-                'avg_ms': dom_ms, 'flop_per_launch': dom_fl}
+                'unit': 'TFLOP/s', 'frac': tf(dom_fl, dom_ms) / PEAK_BF16_TFLOPS,
+                'traffic': HBM_BYTES_PER_LAUNCH.get(dom), 'avg_ms': dom_ms, 'flop_per_launch': dom_fl}
 
     out = {
         'metric': 'attn fwd/bwd TFLOPS and % bf16 MFMA peak, B4 H32 S4096 D128 causal, 1 GPU',
