@@ -223,6 +223,7 @@ void fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[mb][i] = 0.f;
     // S^T = K Q^T with the K operands read one k-step ahead of their MFMAs
+    __builtin_amdgcn_s_setprio(2);
     op_t ka[2][MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) ka[0][mb] = *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR);
@@ -237,6 +238,7 @@ void fwd_kernel(const FwdArgs a) {
       for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(ka[k & 1][mb], qreg[k], s[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
     // first V^T operands: in flight while the softmax runs
     op_t va[2][DB];
 #pragma unroll
@@ -330,6 +332,7 @@ void fwd_kernel(const FwdArgs a) {
         for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
     }
     __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       if (t + 1 < TS) {
@@ -341,6 +344,7 @@ void fwd_kernel(const FwdArgs a) {
       for (int db = 0; db < DB; ++db) o[db] = Tr::mfma(va[t & 1][db], pb[t], o[db]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
   };
 
   // ---- main loop: LDS double buffer, one barrier per tile ---------------------
