@@ -66,6 +66,9 @@ struct BwdArgs {
   MaskArgs mask;
   DropoutArgs drop;
   int32_t num_m_tiles, num_n_tiles;
+  int32_t num_zh;        // (batch or sequences) x heads of the launched kernel's grid
+  int32_t zh_per_xcd;    // ceil(num_zh / 8)
+  int32_t zh_group;      // heads walked together on one XCD
 };
 
 struct EncodedSoftmaxArgs {

@@ -190,55 +190,76 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     ltr_off[i] = (uint32_t)(r * TSTR + cc * 8);
   }
 
-  auto load_tile = [&](int it) {
-    const int hq = hk * group + it / ntq;
-    const int m0 = (br.lo + it % ntq) * BM;
-    const T* qb = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)hq * a.sq.h +
-                  (int64_t)(si.q_start + m0) * a.sq.s;
-    const T* dob = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
-                   (int64_t)hq * a.sdo.h + (int64_t)(si.q_start + m0) * a.sdo.s;
-    const T* ob = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z +
-                  (int64_t)hq * a.so.h + (int64_t)(si.q_start + m0) * a.so.s;
+  // Tile base pointers advance incrementally (one 64-bit add per tensor and tile);
+  // with one wave per SIMD a chain of scalar multiplies per tile is not hidden.
+  const int64_t q_tile_step = (int64_t)BM * a.sq.s, do_tile_step = (int64_t)BM * a.sdo.s,
+                o_tile_step = (int64_t)BM * a.so.s;
+  const T* qb = nullptr; const T* dob = nullptr; const T* ob = nullptr;
+  const float* lse_b = nullptr; const float* delta_b = nullptr;
+  auto set_head = [&](int g) {
+    const int hq = hk * group + g;
+    const int64_t row0 = (int64_t)si.q_start + (int64_t)br.lo * BM;
+    qb = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)hq * a.sq.h + row0 * a.sq.s;
+    dob = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z + (int64_t)hq * a.sdo.h +
+          row0 * a.sdo.s;
+    if (kInlineDelta)
+      ob = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)hq * a.so.h +
+           row0 * a.so.s;
+    lse_b = a.lse + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
+    if (!kInlineDelta) delta_b = a.delta + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
+  };
+  // (g, e) = (q-head inside the GQA group, Q tile inside the range) of the tile to fetch;
+  // called for consecutive tiles only
+  auto load_tile = [&](int g, int e) {
+    if (e == 0) set_head(g);
+    const int m0 = (br.lo + e) * BM;
     const int nvalid = si.seqlen_q - m0;          // > 0
     const bool full = nvalid >= BM;
+    op_t och[CH];
+    if (full) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
-      op_t qv, dv_, ov;
-      if (full) {
-        qv = *reinterpret_cast<const op_t*>(qb + qoff[i]);
-        dv_ = *reinterpret_cast<const op_t*>(dob + dooff[i]);
-        if (kInlineDelta) ov = *reinterpret_cast<const op_t*>(ob + ooff[i]);
-      } else {
-        // ragged last Q tile: rows past the end are zero (they are also masked)
+      for (int i = 0; i < CH; ++i) {
+        if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
+        qch[i] = *reinterpret_cast<const op_t*>(qb + qoff[i]);
+        doch[i] = *reinterpret_cast<const op_t*>(dob + dooff[i]);
+        if (kInlineDelta) och[i] = *reinterpret_cast<const op_t*>(ob + ooff[i]);
+      }
+    } else {
+      // ragged last Q tile: rows past the end are zero (they are also masked)
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
         const bool ok = crow[i] < nvalid;
         const int r = ok ? crow[i] : nvalid - 1;
         const int cc8 = (tid + i * NT) % LPR * 8;
-        qv = *reinterpret_cast<const op_t*>(qb + (int64_t)r * a.sq.s + cc8);
-        dv_ = *reinterpret_cast<const op_t*>(dob + (int64_t)r * a.sdo.s + cc8);
-        if (kInlineDelta) ov = *reinterpret_cast<const op_t*>(ob + (int64_t)r * a.so.s + cc8);
+        op_t qv = *reinterpret_cast<const op_t*>(qb + (int64_t)r * a.sq.s + cc8);
+        op_t dv_ = *reinterpret_cast<const op_t*>(dob + (int64_t)r * a.sdo.s + cc8);
+        if (kInlineDelta) och[i] = *reinterpret_cast<const op_t*>(ob + (int64_t)r * a.so.s + cc8);
         if (!ok) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) { qv[e] = 0; dv_[e] = 0; }
         }
+        qch[i] = qv;
+        doch[i] = dv_;
       }
-      qch[i] = qv;
-      doch[i] = dv_;
-      if (kInlineDelta) {
-        // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310)
+    }
+    if (kInlineDelta) {
+      // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310)
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
         float acc = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dv_[e];
+        for (int e = 0; e < 8; ++e) acc += (float)och[i][e] * (float)doch[i][e];
         dpart[i] = acc;
       }
     }
     if (tid < BM) {
-      const int m = m0 + tid;
-      const bool ok = m < si.seqlen_q;
-      const int64_t lo = lse_offset(si, hq, a.hq) + (ok ? m : 0);
-      l_stage = ok ? a.lse[lo] * kRcpLn2 : 0.f;          // bwd_inner_dk_dv.py:185-186
-      if (!kInlineDelta) d_stage = ok ? a.delta[lo] : 0.f;
+      const bool ok = m0 + tid < si.seqlen_q;
+      l_stage = ok ? lse_b[tid] * kRcpLn2 : 0.f;          // bwd_inner_dk_dv.py:185-186
+      if (!kInlineDelta) d_stage = ok ? delta_b[tid] : 0.f;
     }
+    qb += q_tile_step; dob += do_tile_step; lse_b += BM;
+    if (kInlineDelta) ob += o_tile_step; else delta_b += BM;
   };
 
   auto store_tile = [&](int stage) {
@@ -271,10 +292,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   };
 
   // ---- one (q-head, Q tile) step -----------------------------------------------
-  auto compute = [&](auto masked_tag, int it, int stage) {
+  auto compute = [&](auto masked_tag, int g, int e, int stage) {
     constexpr bool masked = decltype(masked_tag)::value;
-    const int hq = hk * group + it / ntq;
-    const int m0 = (br.lo + it % ntq) * BM;
+    const int hq = hk * group + g;
+    const int m0 = (br.lo + e) * BM;
     char* sp = stage_ptr(stage);
     const T* Qs = reinterpret_cast<const T*>(sp) + c * RSTR + hi * 8;
     const T* dOs = reinterpret_cast<const T*>(sp) + SM::ROW_ELEMS + c * RSTR + hi * 8;
@@ -287,6 +308,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     op_t xa[2][MB];
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR);
 #pragma unroll
@@ -313,6 +335,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], vreg[k], k == 0 ? zero16 : dp[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
     // first transposed operands in flight during the elementwise part
     op_t ta[2][DB];
 #pragma unroll
@@ -368,6 +391,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       sb[t] = pack8<T>(dp[t / 2], t % 2);
     }
     __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       if (t + 1 < TS) {
@@ -392,9 +416,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int db = 0; db < DB; ++db) dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
   };
 
-  load_tile(0);
+  load_tile(0, 0);
   store_tile(0);
   __syncthreads();
   // Per q-head the Q tiles come as [masked | full | masked]; each run has its own
@@ -402,13 +427,17 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   const int n_lb = br.fb_lo <= br.fb_hi ? br.fb_lo - br.lo : ntq;
   const int n_fb = br.fb_lo <= br.fb_hi ? br.fb_hi - br.fb_lo + 1 : 0;
   int it = 0;
+  int g_cur = 0, e_cur = 0;
   auto step = [&](auto masked_tag) {
     const int stage = it & 1;
-    if (it + 1 < total) load_tile(it + 1);
-    compute(masked_tag, it, stage);
+    int g_nxt = g_cur, e_nxt = e_cur + 1;
+    if (e_nxt == ntq) { e_nxt = 0; ++g_nxt; }
+    if (it + 1 < total) load_tile(g_nxt, e_nxt);
+    compute(masked_tag, g_cur, e_cur, stage);
     if (it + 1 < total) store_tile(stage ^ 1);
     __syncthreads();
     ++it;
+    g_cur = g_nxt; e_cur = e_nxt;
   };
   for (int g = 0; g < group; ++g) {
     for (int e = 0; e < n_lb; ++e) step(std::true_type{});
@@ -607,6 +636,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     f32x16 s[MB], dp[MB];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     op_t xa[2][MB];
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR);
 #pragma unroll
@@ -633,6 +663,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], doreg[k], k == 0 ? zero16 : dp[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
     op_t ta[2][DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Kt + db * 32, TSTR);
@@ -673,6 +704,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 #pragma unroll
     for (int t = 0; t < TS; ++t) sb[t] = pack8<T>(dp[t / 2], t % 2);
     __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       if (t + 1 < TS) {
@@ -684,6 +716,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       for (int db = 0; db < DB; ++db) dq[db] = Tr::mfma(ta[t & 1][db], sb[t], dq[db]);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
   };
 
   load_tile(br.lo);
@@ -729,17 +762,31 @@ template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kD
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dkdv_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  const int hk = xcd_remap_head(blockIdx.x, a.hk);
-  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false>(a, hk, blockIdx.y, blockIdx.z, smem_raw);
+  // 1-D grid: each XCD owns a contiguous range of (batch, kv-head) pairs and walks
+  // them in pairs, K tiles in ascending order (the heaviest causal tile first), so the
+  // Q/dO stream of the heads in flight stays in that XCD's L2.
+  const int xcd = blockIdx.x % kNumXcd, li = blockIdx.x / kNumXcd;
+  const int per_group = a.zh_group * a.num_n_tiles;
+  const int gi = li / per_group, gr = li % per_group;
+  const int zl = gi * a.zh_group + gr % a.zh_group;
+  const int zh = xcd * a.zh_per_xcd + zl;
+  if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
+  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false>(a, zh % a.hk, gr / a.zh_group, zh / a.hk, smem_raw);
 }
 
 template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dq_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  const int h = xcd_remap_head(blockIdx.x, a.hq);
-  const int mt = a.num_m_tiles - 1 - (int)blockIdx.y;
-  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, h, mt, blockIdx.z, smem_raw);
+  // same walk as the forward kernel: (batch, q-head) pairs per XCD, heaviest Q tile first
+  const int xcd = blockIdx.x % kNumXcd, li = blockIdx.x / kNumXcd;
+  const int per_group = a.zh_group * a.num_m_tiles;
+  const int gi = li / per_group, gr = li % per_group;
+  const int zl = gi * a.zh_group + gr % a.zh_group;
+  const int zh = xcd * a.zh_per_xcd + zl;
+  if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
+  const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
+  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, zh % a.hq, mt, zh / a.hq, smem_raw);
 }
 
 // grid.y = num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
@@ -804,7 +851,10 @@ hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dro
   constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = NW * 32;
   BwdArgs a = a0;
   a.num_n_tiles = (a.seq.max_seqlen_k + BN - 1) / BN;
-  dim3 grid(a.hk, a.num_n_tiles, bwd_nseq(a));
+  a.num_zh = bwd_nseq(a) * a.hk;
+  a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
+  a.zh_group = 2;
+  dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles));
 #define FA_CALL(W, B, P) launch_with_lds(bwd_dkdv_kernel<T, D, NW, BM, W, B, P>, grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
@@ -815,7 +865,10 @@ hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropo
   constexpr int NW = BwdTile<D>::NW, BN = BwdTile<D>::DQ_BN, BM = NW * 32;
   BwdArgs a = a0;
   a.num_m_tiles = (a.seq.max_seqlen_q + BM - 1) / BM;
-  dim3 grid(a.hq, a.num_m_tiles, bwd_nseq(a));
+  a.num_zh = bwd_nseq(a) * a.hq;
+  a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
+  a.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
+  dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_m_tiles));
 #define FA_CALL(W, B, P) launch_with_lds(bwd_dq_kernel<T, D, NW, BN, W, B, P>, grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
