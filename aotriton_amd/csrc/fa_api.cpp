@@ -315,7 +315,6 @@ int fa_validate_bwd(const fa_bwd_params* params, int32_t params_version, const f
 }
 
 int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_config* out) {
-  (void)num_cu;
   if (out == nullptr) return FA_ERROR_INVALID_VALUE;
   Shape s{};
   int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
@@ -329,7 +328,11 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
     const int ratio = s.hq / s.hk;
     const int zg = ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2;
     const int groups = (zh_per_xcd + zg - 1) / zg;
-    out->grid[0] = fa::kNumXcd * groups * zg * ((s.max_sq + t.block_m - 1) / t.block_m);
+    // persistent workgroups: one per CU, at most one per Q tile
+    const int items = groups * zg * ((s.max_sq + t.block_m - 1) / t.block_m);
+    int workers = (num_cu > 0 ? num_cu : 256) / fa::kNumXcd;
+    workers = workers < 1 ? 1 : (workers > items ? items : workers);
+    out->grid[0] = fa::kNumXcd * workers;
     out->grid[1] = 1;
     out->grid[2] = 1;
   }
@@ -411,6 +414,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
   a.seed_out = static_cast<uint64_t*>(p->philox_seed_output.ptr);
   a.offset_out = static_cast<uint64_t*>(p->philox_offset_output.ptr);
   a.atomic_counter = static_cast<int32_t*>(p->persistent_atomic_counter.ptr);
+  a.num_cu = dev->num_cu;
 
   const fa::TileShape t = fa::fwd_tile_shape(s.d);
   FA_LOG(4, "attn_fwd: D=%d BLOCK_M=%d BLOCK_N=%d waves=%d lds=%d windowed=%d bias=%d dropout=%d nseq=%d",

@@ -46,10 +46,12 @@ struct FwdArgs {
   DropoutArgs drop;
   uint64_t* seed_out; uint64_t* offset_out;
   int32_t* atomic_counter;
+  int32_t num_cu;        // CUs of the device (host fills it in)
   int32_t num_m_tiles;
   int32_t num_zh;        // (batch or sequences) x q-heads
   int32_t zh_per_xcd;    // ceil(num_zh / 8)
   int32_t zh_group;      // heads walked together on one XCD
+  int32_t items_per_xcd; // Q tiles (incl. padding of the last group) per XCD
 };
 
 struct BwdArgs {

@@ -551,7 +551,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc += (float)o8[e] * (float)doreg[k][e];
     }
-    d_row = acc + xor32(acc);
+    d_row = cross_sum(acc);
   } else {
     d_row = a.delta[lo];
   }

@@ -128,7 +128,26 @@ __device__ __forceinline__ void scale_acc(f32x16& acc, float f) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+// Reductions across the two halves of a wave (lane <-> lane ^ 32) with
+// v_permlane32_swap: after the swap one register holds the lower half's value in
+// both halves and the other one the upper half's value; no LDS round trip.
+__device__ __forceinline__ void wave_halves(float x, float& lower, float& upper) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  lower = __builtin_bit_cast(float, r0);
+  upper = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float cross_max(float x) {
+  float lo, up;
+  wave_halves(x, lo, up);
+  return fmaxf(lo, up);
+}
+__device__ __forceinline__ float cross_sum(float x) {
+  float lo, up;
+  wave_halves(x, lo, up);
+  return lo + up;
+}
 
 // Philox-4x32-10 with counter (c0, c1, 0, 0); Salmon et al. SC'11.  The
 // reference reaches it through Triton's tl.randint4x

@@ -30,10 +30,9 @@ struct FwdSmem {
   static constexpr int BYTES = STAGES * (K_ELEMS + V_ELEMS) * 2;
 };
 
+// One Q tile (BM rows of head h of sequence z) against all its visible K/V tiles.
 template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
-__global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
-__attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1, D <= 128 ? 2 : 1)))
-void fwd_kernel(const FwdArgs a) {
+__device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const int h, const int mt, char* smem_raw) {
   using Tr = Traits<T>;
   using op_t = typename Tr::op_t;
   using q4_t = typename Tr::q4_t;
@@ -48,37 +47,11 @@ void fwd_kernel(const FwdArgs a) {
   constexpr int CH = (BN * D / 8) / NT;                   // 16-byte chunks per thread, per tensor
   static_assert((BN * D / 8) % NT == 0, "tile must split evenly");
 
-  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   T* Ks = reinterpret_cast<T*>(smem_raw);
   T* Vs = Ks + SM::STAGES * SM::K_ELEMS;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-
-  // 1-D grid.  Consecutive workgroup ids round-robin over the 8 XCDs; each XCD walks
-  // its own contiguous range of (batch, head) pairs in small groups: inside a group
-  // the Q tiles go heaviest-first (causal) with the heads of the group interleaved.
-  // Few heads are in flight per XCD, so their K/V stay in that XCD's L2, and the
-  // stream of groups keeps the CUs of the XCD evenly loaded.
-  const int xcd = blockIdx.x % kNumXcd;
-  const int li = blockIdx.x / kNumXcd;
-  const int per_group = a.zh_group * a.num_m_tiles;
-  const int gi = li / per_group, gr = li % per_group;
-  const int zh_local = gi * a.zh_group + gr % a.zh_group;
-  const int zh = xcd * a.zh_per_xcd + zh_local;
-  if (zh_local >= a.zh_per_xcd || zh >= a.num_zh) return;
-  const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
-  const int z = zh / a.hq;
-  const int h = zh % a.hq;
-
-  if (kDropout && blockIdx.x == 0 && tid == 0) {
-    // modules/flash/kernel/fwd_kernel.py:199-207
-    const uint64_t seed = *a.drop.seed_ptr;
-    uint64_t base = a.drop.offset2;
-    if (a.drop.offset1_ptr) base += *a.drop.offset1_ptr;
-    if (a.seed_out) *a.seed_out = seed;
-    if (a.offset_out) *a.offset_out = base;
-  }
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * BM;
@@ -134,56 +107,42 @@ void fwd_kernel(const FwdArgs a) {
   if (kDropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
 
   // ---- global -> register -> LDS staging -------------------------------------
-  // Thread-constant offsets inside a tile; the tile base is wave-uniform.
+  // Buffer loads: the descriptor is rebased on every tile and bounds the tile to its
+  // valid rows, so rows past the end of the sequence read as zero (their scores are
+  // masked and P is 0 there) and no per-lane address arithmetic is needed: a thread's
+  // chunks sit RPI rows apart, which is a scalar offset on the global side and an
+  // immediate offset on the LDS side.
+  constexpr int LPR = D / 8;              // 16-byte chunks per row
+  constexpr int RPI = NT / LPR;           // rows between two chunks of one thread
+  static_assert(NT % LPR == 0, "threads must cover whole rows");
   op_t kreg[CH], vreg[CH];
-  uint32_t koff[CH], voff[CH];
-  int lrow[CH];
-  uint32_t ldsk[CH], ldsv[CH];
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int idx = tid + i * NT;
-    const int r = idx / (D / 8), cc = idx % (D / 8);
-    lrow[i] = r;
-    koff[i] = (uint32_t)(r * (int)a.sk.s + cc * 8);
-    voff[i] = (uint32_t)(r * (int)a.sv.s + cc * 8);
-    ldsk[i] = (uint32_t)(r * KSTR + cc * 8);
-    ldsv[i] = (uint32_t)(r * VSTR + cc * 8);
-  }
+  const int r0 = tid / LPR, cc0 = tid % LPR;
+  const int kvoff = r0 * (int)a.sk.s * 2 + cc0 * 16;      // bytes inside a tile
+  const int vvoff = r0 * (int)a.sv.s * 2 + cc0 * 16;
+  const int ksoff = RPI * (int)a.sk.s * 2, vsoff = RPI * (int)a.sv.s * 2;
+  const int ldsk0 = r0 * KSTR + cc0 * 8, ldsv0 = r0 * VSTR + cc0 * 8;   // elements
 
   auto load_tile = [&](int j) {
-    const T* kt = kbase + (int64_t)j * BN * a.sk.s;
-    const T* vt = vbase + (int64_t)j * BN * a.sv.s;
-    if ((j + 1) * BN <= si.seqlen_k) {
+    const int rows = si.seqlen_k - j * BN < BN ? si.seqlen_k - j * BN : BN;    // > 0
+    const auto krs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(kbase + (int64_t)j * BN * a.sk.s), 0, ((rows - 1) * (int)a.sk.s + D) * 2, 0x00020000);
+    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(vbase + (int64_t)j * BN * a.sv.s), 0, ((rows - 1) * (int)a.sv.s + D) * 2, 0x00020000);
 #pragma unroll
-      for (int i = 0; i < CH; ++i) kreg[i] = *reinterpret_cast<const op_t*>(kt + koff[i]);
+    for (int i = 0; i < CH; ++i)
+      kreg[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvoff, i * ksoff, 0));
 #pragma unroll
-      for (int i = 0; i < CH; ++i) vreg[i] = *reinterpret_cast<const op_t*>(vt + voff[i]);
-    } else {
-      // ragged last tile: rows past the end are clamped (K) / zeroed (V: P is 0 there)
-      const int nvalid = si.seqlen_k - j * BN;
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const bool ok = lrow[i] < nvalid;
-        const int cc8 = (tid + i * NT) % (D / 8) * 8;
-        const int r = ok ? lrow[i] : nvalid - 1;
-        kreg[i] = *reinterpret_cast<const op_t*>(kt + (int64_t)r * a.sk.s + cc8);
-        op_t x = *reinterpret_cast<const op_t*>(vt + (int64_t)r * a.sv.s + cc8);
-        if (!ok) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = 0;
-        }
-        vreg[i] = x;
-      }
-    }
+    for (int i = 0; i < CH; ++i)
+      vreg[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(vrs, vvoff, i * vsoff, 0));
   };
 
   auto store_tile = [&](int stage) {
-    T* ks = Ks + stage * SM::K_ELEMS;
-    T* vs = Vs + stage * SM::V_ELEMS;
+    T* ks = Ks + stage * SM::K_ELEMS + ldsk0;
+    T* vs = Vs + stage * SM::V_ELEMS + ldsv0;
 #pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<op_t*>(ks + ldsk[i]) = kreg[i];
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<op_t*>(ks + i * RPI * KSTR) = kreg[i];
 #pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<op_t*>(vs + ldsv[i]) = vreg[i];
+    for (int i = 0; i < CH; ++i) *reinterpret_cast<op_t*>(vs + i * RPI * VSTR) = vreg[i];
   };
 
   // ---- online softmax state --------------------------------------------------
@@ -214,31 +173,39 @@ void fwd_kernel(const FwdArgs a) {
     wave_hi = cmax < 0 ? -1 : (int)(cmax / BN);
   }
 
-  auto compute = [&](int j, int stage, bool masked) {
+  f32x16 s[MB];   // S^T of the current tile
+
+  auto qk = [&](int stage) {
     const T* ks = Ks + stage * SM::K_ELEMS + c * KSTR + hi * 8;
-    const T* vs = Vs + stage * SM::V_ELEMS + v_lane;
-    f32x16 s[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[mb][i] = 0.f;
-    // S^T = K Q^T with the K operands read one k-step ahead of their MFMAs
+    // S^T = K Q^T with the K operands read kAhead k-steps ahead of their MFMAs
     __builtin_amdgcn_s_setprio(2);
-    op_t ka[2][MB];
+    constexpr int kAhead = 2;
+    op_t ka[kAhead + 1][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) ka[0][mb] = *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR);
+    for (int k = 0; k < kAhead; ++k)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) ka[k][mb] = *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR + k * 16);
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
-      if (k + 1 < KS) {
+      if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          ka[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR + (k + 1) * 16);
+          ka[(k + kAhead) % (kAhead + 1)][mb] =
+              *reinterpret_cast<const op_t*>(ks + mb * 32 * KSTR + (k + kAhead) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(ka[k & 1][mb], qreg[k], s[mb]);
+      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(ka[k % (kAhead + 1)][mb], qreg[k], s[mb]);
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_s_setprio(0);
+  };
+
+  auto sv = [&](int j, int stage, bool masked) {
+    const T* vs = Vs + stage * SM::V_ELEMS + v_lane;
     // first V^T operands: in flight while the softmax runs
     op_t va[2][DB];
 #pragma unroll
@@ -276,7 +243,7 @@ void fwd_kernel(const FwdArgs a) {
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
-    mx = fmaxf(mx, xor32(mx));
+    mx = cross_max(mx);
     // Lazy rescaling: a row adopts the new maximum only when it grew by more than
     // 2^8 in the exponent domain; until then p may exceed 1 (at most 256), which
     // fp32 accumulation and the 16-bit P operand absorb, and the final O = acc / l
@@ -354,13 +321,16 @@ void fwd_kernel(const FwdArgs a) {
   for (int j = br.lo; j <= br.hi; ++j) {
     const int stage = (j - br.lo) & 1;
     if (j < br.hi) load_tile(j + 1);
-    if (j <= wave_hi) compute(j, stage, !br.is_full(j));
+    if (j <= wave_hi) {
+      qk(stage);
+      sv(j, stage, !br.is_full(j));
+    }
     if (j < br.hi) store_tile(stage ^ 1);
     __syncthreads();
   }
 
   // ---- epilogue ----------------------------------------------------------------
-  const float l = l_i + xor32(l_i);
+  const float l = cross_sum(l_i);
   const bool alive = l > 0.f;
   float inv = alive ? 1.0f / l : 0.f;
   if (kDropout) inv *= ds.scale;          // fwd_kernel.py:573-575
@@ -376,6 +346,44 @@ void fwd_kernel(const FwdArgs a) {
       }
     if (lse_ptr && hi == 0)
       lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
+  }
+}
+
+// Persistent workgroups: the grid holds one workgroup per CU.  Consecutive workgroup
+// ids round-robin over the 8 XCDs; each XCD owns a contiguous range of (batch, head)
+// pairs, so the K/V of a head stay in one L2.  The Q tiles of an XCD are ordered in
+// small groups of heads, inside a group heaviest-first (causal) with the heads
+// interleaved, and the workgroups of the XCD take them in serpentine order (worker p
+// takes p, 2P-1-p, 2P+p, ...), which pairs heavy with light tiles.  A workgroup
+// goes from one tile to the next without a relaunch.
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
+__global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
+__attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1, D <= 128 ? 2 : 1)))
+void fwd_kernel(const FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  if (kDropout && blockIdx.x == 0 && threadIdx.x == 0) {
+    // modules/flash/kernel/fwd_kernel.py:199-207
+    const uint64_t seed = *a.drop.seed_ptr;
+    uint64_t base = a.drop.offset2;
+    if (a.drop.offset1_ptr) base += *a.drop.offset1_ptr;
+    if (a.seed_out) *a.seed_out = seed;
+    if (a.offset_out) *a.offset_out = base;
+  }
+  const int xcd = blockIdx.x % kNumXcd;
+  const int p = blockIdx.x / kNumXcd;
+  const int workers = gridDim.x / kNumXcd;
+  const int per_group = a.zh_group * a.num_m_tiles;
+  const int items = a.items_per_xcd;
+  for (int r = 0;; ++r) {
+    const int t = r * workers + ((r & 1) ? workers - 1 - p : p);
+    if (r * workers >= items) break;
+    if (t >= items) continue;
+    const int gi = t / per_group, gr = t % per_group;
+    const int zh_local = gi * a.zh_group + gr % a.zh_group;
+    const int zh = xcd * a.zh_per_xcd + zh_local;
+    if (zh_local >= a.zh_per_xcd || zh >= a.num_zh) continue;
+    const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
+    fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout>(a, zh / a.hq, zh % a.hq, mt, smem_raw);
   }
 }
 
@@ -410,7 +418,11 @@ hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, 
   b.zh_per_xcd = (b.num_zh + kNumXcd - 1) / kNumXcd;
   b.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
   const int groups = (b.zh_per_xcd + b.zh_group - 1) / b.zh_group;
-  dim3 grid((unsigned)(kNumXcd * groups * b.zh_group * b.num_m_tiles));
+  b.items_per_xcd = groups * b.zh_group * b.num_m_tiles;
+  int workers = a.num_cu / kNumXcd;          // one workgroup per CU
+  if (workers < 1) workers = 1;
+  if (workers > b.items_per_xcd) workers = b.items_per_xcd;
+  dim3 grid((unsigned)(kNumXcd * workers));
   const int key = (windowed ? 4 : 0) | (bias ? 2 : 0) | (dropout ? 1 : 0);
   switch (key) {
     case 0: return launch_fwd_variant<T, D, false, false, false>(b, grid, stream);

@@ -123,7 +123,7 @@ def test_validate_fwd_error_contract():
     p, keep = _fwd_params()
     err, cfg = query_fwd_config(p)
     assert err == E.hipSuccess and cfg.block_m == 256 and cfg.head_dim == 128
-    assert list(cfg.grid) == [16, 1, 1]     # 8 XCDs x one group of 2 head slots x 1 Q tile
+    assert list(cfg.grid) == [16, 1, 1]     # persistent workgroups: 8 XCDs x min(CUs per XCD, 2 Q-tile slots per XCD)
 
 
 def test_validate_bwd_error_contract():
