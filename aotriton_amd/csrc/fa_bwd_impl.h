@@ -307,40 +307,6 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     f32x16 s[MB], dp[MB];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    op_t xa[2][MB];
-    __builtin_amdgcn_s_setprio(2);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR);
-#pragma unroll
-    for (int k = 0; k < KS; ++k) {
-      if (k + 1 < KS) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + (k + 1) * 16);
-      }
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], kreg[k], k == 0 ? zero16 : s[mb]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR);
-#pragma unroll
-    for (int k = 0; k < KS; ++k) {
-      if (k + 1 < KS) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + (k + 1) * 16);
-      }
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], vreg[k], k == 0 ? zero16 : dp[mb]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __builtin_amdgcn_s_setprio(0);
-    // first transposed operands in flight during the elementwise part
-    op_t ta[2][DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(dOt + db * 32, TSTR);
-
     DropoutState dst{};
     if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
     const T* bptr = nullptr;
@@ -348,61 +314,162 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)hq * a.sb_h +
              (int64_t)key_c * a.sb_n;
 
+    // The vector ALU work is spread over the MFMAs of the GEMMs that do not depend on
+    // it: p = exp2(...) of S runs behind the MFMAs of dP, ds = p (dP - delta) behind
+    // those of dV.  Fences keep the hand-made order.
+    constexpr int kAhead = 2;
+    op_t xa[kAhead + 1][MB];
+    op_t pb[TS], sb[TS];
+    f32x4 l4[MB][4], d4[MB][4];
+
+    // ---- S = Q K^T ---------------------------------------------------------------
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + k * 16);
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k + kAhead < KS) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          xa[(k + kAhead) % (kAhead + 1)][mb] =
+              *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + (k + kAhead) * 16);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kreg[k], k == 0 ? zero16 : s[mb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // row statistics of the tile's queries and the first dO operands
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int mloc = 32 * mb + 8 * g + 4 * hi;
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Ls + mloc);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Ds + mloc);
+      for (int g = 0; g < 4; ++g) l4[mb][g] = *reinterpret_cast<const f32x4*>(Ls + 32 * mb + 8 * g + 4 * hi);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = 4 * g + r;
-          const int m = m0 + mloc + r;
-          // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
-          float x;
-          if (kBias) {
-            const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
-            x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)mm * a.sb_m] * kLog2e) - l4[r];
-          } else {
-            x = __builtin_fmaf(s[mb][i], qk_scale, -l4[r]);
-          }
-          if (masked) {
-            bool vis = (m < si.seqlen_q) & key_ok;
-            if (kWindowed) vis = vis & (key <= m + w.right) & (key >= m - w.left);
-            x = vis ? x : -__builtin_inff();
-          }
-          const float p = fast_exp2(x);
-          float pd = p, dpv = dp[mb][i];
-          if (kDropout) {
-            const bool keep = dropout_keep1(dst, m, key);
-            pd = keep ? p * dst.scale : 0.f;              // :200-201
-            dpv = keep ? dpv * dst.scale : 0.f;           // :239-240
-          }
-          s[mb][i] = pd;
-          dp[mb][i] = p * (dpv - d4[r]);                  // ds uses the undropped p (:242)
-        }
-      }
+    for (int k = 0; k < kAhead; ++k)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + k * 16);
 
-    op_t pb[TS], sb[TS];
+    // element E = 16*mb + i of the tile: p (kept in s, undropped) and its operand form
+    auto p_el = [&](int E) {
+      const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
+      const int m = m0 + 32 * mb + 8 * g + 4 * hi + r;
+      // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
+      float x;
+      if (kBias) {
+        const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
+        x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)mm * a.sb_m] * kLog2e) - l4[mb][g][r];
+      } else {
+        x = __builtin_fmaf(s[mb][i], qk_scale, -l4[mb][g][r]);
+      }
+      if (masked) {
+        bool vis = (m < si.seqlen_q) & key_ok;
+        if (kWindowed) vis = vis & (key <= m + w.right) & (key >= m - w.left);
+        x = vis ? x : -__builtin_inff();
+      }
+      s[mb][i] = fast_exp2(x);
+    };
+    bool keep_bit[kDropout ? 16 * MB : 1];
+    auto p_pair = [&](int E) {   // E odd: operand form of (E-1, E); dropout applies to the operand only
+      float p0 = s[E / 16][E % 16 - 1], p1 = s[E / 16][E % 16];
+      if (kDropout) {
+        const int mb = E / 16;
 #pragma unroll
-    for (int t = 0; t < TS; ++t) {
-      pb[t] = pack8<T>(s[t / 2], t % 2);     // p cast to dO's dtype, ds to Q's (composed_tensors.py:191-193)
-      sb[t] = pack8<T>(dp[t / 2], t % 2);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(2);
+        for (int q = 0; q < 2; ++q) {
+          const int i = E % 16 - 1 + q;
+          const int m = m0 + 32 * mb + 8 * (i / 4) + 4 * hi + (i % 4);
+          keep_bit[E - 1 + q] = dropout_keep1(dst, m, key);
+        }
+        p0 = keep_bit[E - 1] ? p0 * dst.scale : 0.f;              // :200-201
+        p1 = keep_bit[E] ? p1 * dst.scale : 0.f;
+      }
+      pb[E / 8][E % 8 - 1] = Tr::cvt(p0);     // p cast to dO's dtype (composed_tensors.py:191-193)
+      pb[E / 8][E % 8] = Tr::cvt(p1);
+    };
+    auto ds_el = [&](int E) {
+      const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
+      float dpv = dp[mb][i];
+      if (kDropout) dpv = keep_bit[E] ? dpv * dst.scale : 0.f;   // :239-240
+      dp[mb][i] = s[mb][i] * (dpv - d4[mb][g][r]);                // ds uses the undropped p (:242)
+    };
+    auto ds_pair = [&](int E) {  // E odd: ds cast to Q's dtype
+      sb[E / 8][E % 8 - 1] = Tr::cvt(dp[E / 16][E % 16 - 1]);
+      sb[E / 8][E % 8] = Tr::cvt(dp[E / 16][E % 16]);
+    };
+
+    // ---- dP = dO V^T, with p behind its MFMAs ------------------------------------
+    constexpr int EPG1 = 16 * MB / (KS * MB);    // elements per MFMA (D = 128: 2)
+    static_assert(16 * MB % (KS * MB) == 0 || KS * MB > 16 * MB, "element split");
 #pragma unroll
-    for (int t = 0; t < TS; ++t) {
-      if (t + 1 < TS) {
+    for (int k = 0; k < KS; ++k) {
+      if (k + kAhead < KS) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = lds_read_tr8<T>(dOt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+        for (int mb = 0; mb < MB; ++mb)
+          xa[(k + kAhead) % (kAhead + 1)][mb] =
+              *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + (k + kAhead) * 16);
       }
 #pragma unroll
-      for (int db = 0; db < DB; ++db) dv[db] = Tr::mfma(ta[t & 1][db], pb[t], dv[db]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int mb = 0; mb < MB; ++mb) {
+        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], vreg[k], k == 0 ? zero16 : dp[mb]);
+        const int gidx = k * MB + mb;
+        if (EPG1 >= 1) {
+#pragma unroll
+          for (int e = 0; e < (EPG1 >= 1 ? EPG1 : 1); ++e) {
+            const int E = gidx * EPG1 + e;
+            p_el(E);
+            if (E & 1) p_pair(E);
+          }
+        } else {
+          // more MFMAs than elements (D = 256): one element every other MFMA
+          constexpr int every = (KS * MB) / (16 * MB);
+          if (gidx % every == 0) {
+            const int E = gidx / every;
+            p_el(E);
+            if (E & 1) p_pair(E);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
+    // delta of the tile's queries, first transposed dO operands
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) d4[mb][g] = *reinterpret_cast<const f32x4*>(Ds + 32 * mb + 8 * g + 4 * hi);
+    op_t ta[2][DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(dOt + db * 32, TSTR);
+
+    // ---- dV^T += dO^T P, with ds behind its MFMAs --------------------------------
+    constexpr int G3 = TS * DB;
+    constexpr int EPG3 = 16 * MB / G3;           // D = 128: 2
+    static_assert(16 * MB % G3 == 0 || G3 > 16 * MB, "element split");
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        if (t + 1 < TS) ta[(t + 1) & 1][db] = lds_read_tr8<T>(dOt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+        dv[db] = Tr::mfma(ta[t & 1][db], pb[t], dv[db]);
+        const int gidx = t * DB + db;
+        if (EPG3 >= 1) {
+#pragma unroll
+          for (int e = 0; e < (EPG3 >= 1 ? EPG3 : 1); ++e) {
+            const int E = gidx * EPG3 + e;
+            ds_el(E);
+            if (E & 1) ds_pair(E);
+          }
+        } else {
+          constexpr int every = G3 / (16 * MB);
+          if (gidx % every == 0) {
+            const int E = gidx / every;
+            ds_el(E);
+            if (E & 1) ds_pair(E);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- dK^T += Q^T dS ----------------------------------------------------------
 #pragma unroll
     for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Qt + db * 32, TSTR);
 #pragma unroll
@@ -416,7 +483,6 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int db = 0; db < DB; ++db) dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_s_setprio(0);
   };
 
   load_tile(0, 0);

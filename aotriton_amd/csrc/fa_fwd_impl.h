@@ -122,18 +122,26 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   const int ksoff = RPI * (int)a.sk.s * 2, vsoff = RPI * (int)a.sv.s * 2;
   const int ldsk0 = r0 * KSTR + cc0 * 8, ldsv0 = r0 * VSTR + cc0 * 8;   // elements
 
-  auto load_tile = [&](int j) {
-    const int rows = si.seqlen_k - j * BN < BN ? si.seqlen_k - j * BN : BN;    // > 0
-    const auto krs = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T*>(kbase + (int64_t)j * BN * a.sk.s), 0, ((rows - 1) * (int)a.sk.s + D) * 2, 0x00020000);
-    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T*>(vbase + (int64_t)j * BN * a.sv.s), 0, ((rows - 1) * (int)a.sv.s + D) * 2, 0x00020000);
+  // tiles are fetched in ascending order: the tile bases and the count of rows left
+  // advance by one tile per call
+  const T* kt = kbase + (int64_t)br.lo * BN * a.sk.s;
+  const T* vt = vbase + (int64_t)br.lo * BN * a.sv.s;
+  const int64_t k_step = (int64_t)BN * a.sk.s, v_step = (int64_t)BN * a.sv.s;
+  const int k_row_bytes = (int)a.sk.s * 2, v_row_bytes = (int)a.sv.s * 2;
+  int rows_left = si.seqlen_k - br.lo * BN;      // > 0
+  auto load_next_tile = [&]() {
+    const int rows = rows_left < BN ? rows_left : BN;
+    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, (rows - 1) * k_row_bytes + D * 2,
+                                                       0x00020000);
+    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, (rows - 1) * v_row_bytes + D * 2,
+                                                       0x00020000);
 #pragma unroll
     for (int i = 0; i < CH; ++i)
       kreg[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvoff, i * ksoff, 0));
 #pragma unroll
     for (int i = 0; i < CH; ++i)
       vreg[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(vrs, vvoff, i * vsoff, 0));
+    kt += k_step; vt += v_step; rows_left -= BN;
   };
 
   auto store_tile = [&](int stage) {
@@ -315,12 +323,12 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   };
 
   // ---- main loop: LDS double buffer, one barrier per tile ---------------------
-  load_tile(br.lo);
+  load_next_tile();
   store_tile(0);
   __syncthreads();
   for (int j = br.lo; j <= br.hi; ++j) {
     const int stage = (j - br.lo) & 1;
-    if (j < br.hi) load_tile(j + 1);
+    if (j < br.hi) load_next_tile();
     if (j <= wave_hi) {
       qk(stage);
       sv(j, stage, !br.is_full(j));
