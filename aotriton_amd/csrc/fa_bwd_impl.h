@@ -173,22 +173,21 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   auto stage_ptr = [&](int stage) { return smem_raw + stage * SM::STAGE_BYTES; };
 
   // ---- staging -----------------------------------------------------------------
-  op_t qch[CH], doch[CH];
+  // Q and dO tiles travel global -> registers -> LDS in 16-byte pieces.  The pieces
+  // are issued between the MFMAs of the running tile (loads behind S = Q K^T, LDS
+  // writes behind dK^T += Q^T dS), so staging costs no issue time of its own.
+  // Buffer loads with a descriptor rebased on every tile: rows past the end of the
+  // sequence read as zero, and a descriptor of zero records turns the fetch after
+  // the last tile into a no-op.
+  static_assert(NCH % NT == 0, "threads must cover the tile evenly");
+  constexpr int RPI = NT / LPR;                  // rows between two pieces of one thread
+  op_t qch[CH], doch[CH], och[kInlineDelta ? CH : 1];
   float l_stage = 0.f, d_stage = 0.f;
-  float dpart[CH];
-  int crow[CH];
-  uint32_t qoff[CH], dooff[CH], ooff[CH], lrow_off[CH], ltr_off[CH];
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int idx = tid + i * NT;
-    const int r = idx / LPR, cc = idx % LPR;
-    crow[i] = r;
-    qoff[i] = (uint32_t)(r * (int)a.sq.s + cc * 8);
-    dooff[i] = (uint32_t)(r * (int)a.sdo.s + cc * 8);
-    ooff[i] = (uint32_t)(r * (int)a.so.s + cc * 8);
-    lrow_off[i] = (uint32_t)(r * RSTR + cc * 8);
-    ltr_off[i] = (uint32_t)(r * TSTR + cc * 8);
-  }
+  const int r0 = tid / LPR, cc0 = tid % LPR;
+  const int q_voff = r0 * (int)a.sq.s * 2 + cc0 * 16, do_voff = r0 * (int)a.sdo.s * 2 + cc0 * 16,
+            o_voff = r0 * (int)a.so.s * 2 + cc0 * 16;                     // bytes inside a tile
+  const int q_soff = RPI * (int)a.sq.s * 2, do_soff = RPI * (int)a.sdo.s * 2, o_soff = RPI * (int)a.so.s * 2;
+  const int lrow0 = r0 * RSTR + cc0 * 8, ltr0 = r0 * TSTR + cc0 * 8;      // elements
 
   // Tile base pointers advance incrementally (one 64-bit add per tensor and tile);
   // with one wave per SIMD a chain of scalar multiplies per tile is not hidden.
@@ -208,85 +207,75 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     lse_b = a.lse + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
     if (!kInlineDelta) delta_b = a.delta + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
   };
+  __amdgpu_buffer_rsrc_t q_rs, do_rs, o_rs;
   // (g, e) = (q-head inside the GQA group, Q tile inside the range) of the tile to fetch;
-  // called for consecutive tiles only
-  auto load_tile = [&](int g, int e) {
-    if (e == 0) set_head(g);
+  // called for consecutive tiles only; `live` false: nothing is fetched
+  auto fetch_begin = [&](bool live, int g, int e) {
+    if (live && e == 0) set_head(g);
     const int m0 = (br.lo + e) * BM;
-    const int nvalid = si.seqlen_q - m0;          // > 0
-    const bool full = nvalid >= BM;
-    op_t och[CH];
-    if (full) {
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
-        qch[i] = *reinterpret_cast<const op_t*>(qb + qoff[i]);
-        doch[i] = *reinterpret_cast<const op_t*>(dob + dooff[i]);
-        if (kInlineDelta) och[i] = *reinterpret_cast<const op_t*>(ob + ooff[i]);
-      }
-    } else {
-      // ragged last Q tile: rows past the end are zero (they are also masked)
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
-        const bool ok = crow[i] < nvalid;
-        const int r = ok ? crow[i] : nvalid - 1;
-        const int cc8 = (tid + i * NT) % LPR * 8;
-        op_t qv = *reinterpret_cast<const op_t*>(qb + (int64_t)r * a.sq.s + cc8);
-        op_t dv_ = *reinterpret_cast<const op_t*>(dob + (int64_t)r * a.sdo.s + cc8);
-        if (kInlineDelta) och[i] = *reinterpret_cast<const op_t*>(ob + (int64_t)r * a.so.s + cc8);
-        if (!ok) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) { qv[e] = 0; dv_[e] = 0; }
-        }
-        qch[i] = qv;
-        doch[i] = dv_;
-      }
-    }
-    if (kInlineDelta) {
-      // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310)
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        float acc = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)och[i][e] * (float)doch[i][e];
-        dpart[i] = acc;
-      }
-    }
+    int rows = si.seqlen_q - m0 < BM ? si.seqlen_q - m0 : BM;
+    rows = live ? rows : 0;
+    const bool any = rows > 0;
+    q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + D) * 2 : 0,
+                                             0x00020000);
+    do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
+                                              any ? ((rows - 1) * (int)a.sdo.s + D) * 2 : 0, 0x00020000);
+    if (kInlineDelta)
+      o_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ob), 0,
+                                               any ? ((rows - 1) * (int)a.so.s + D) * 2 : 0, 0x00020000);
     if (tid < BM) {
-      const bool ok = m0 + tid < si.seqlen_q;
-      l_stage = ok ? lse_b[tid] * kRcpLn2 : 0.f;          // bwd_inner_dk_dv.py:185-186
+      const bool ok = tid < rows;
+      l_stage = ok ? lse_b[tid] : 0.f;
       if (!kInlineDelta) d_stage = ok ? delta_b[tid] : 0.f;
     }
-    qb += q_tile_step; dob += do_tile_step; lse_b += BM;
-    if (kInlineDelta) ob += o_tile_step; else delta_b += BM;
+    if (live) {
+      qb += q_tile_step; dob += do_tile_step; lse_b += BM;
+      if (kInlineDelta) ob += o_tile_step; else delta_b += BM;
+    }
   };
-
-  auto store_tile = [&](int stage) {
+  constexpr int FETCH_PIECES = 2 * CH;
+  auto fetch_piece = [&](int i) {        // Q pieces first, then dO (and O)
+    if (i < CH) {
+      qch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(q_rs, q_voff, i * q_soff, 0));
+    } else {
+      const int k = i - CH;
+      doch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(do_rs, do_voff, k * do_soff, 0));
+      if (kInlineDelta)
+        och[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(o_rs, o_voff, k * o_soff, 0));
+    }
+  };
+  constexpr int STORE_PIECES = 4 * CH;
+  auto store_piece = [&](int i, int stage) {   // same order as the fetches; two copies each
     char* sp = stage_ptr(stage);
     T* Qs = reinterpret_cast<T*>(sp);
     T* dOs = Qs + SM::ROW_ELEMS;
     T* Qt = dOs + SM::ROW_ELEMS;
     T* dOt = Qt + SM::TR_ELEMS;
-    float* Ls = reinterpret_cast<float*>(dOt + SM::TR_ELEMS);
+    const int tensor = i / (2 * CH), k = (i % (2 * CH)) / 2, copy = i % 2;
+    const op_t v = tensor == 0 ? qch[k] : doch[k];
+    T* dst = copy == 0 ? (tensor == 0 ? Qs : dOs) + lrow0 + k * RPI * RSTR
+                       : (tensor == 0 ? Qt : dOt) + ltr0 + k * RPI * TSTR;
+    *reinterpret_cast<op_t*>(dst) = v;
+  };
+  auto store_stats = [&](int stage) {
+    char* sp = stage_ptr(stage);
+    float* Ls = reinterpret_cast<float*>(reinterpret_cast<T*>(sp) + 2 * SM::ROW_ELEMS + 2 * SM::TR_ELEMS);
     float* Ds = Ls + BM;
+    if (kInlineDelta) {
+      // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310); the LPR threads
+      // that share a row are consecutive lanes
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      if (NCH % NT != 0 && tid + i * NT >= NCH) continue;
-      *reinterpret_cast<op_t*>(Qs + lrow_off[i]) = qch[i];
-      *reinterpret_cast<op_t*>(Qt + ltr_off[i]) = qch[i];
-      *reinterpret_cast<op_t*>(dOs + lrow_off[i]) = doch[i];
-      *reinterpret_cast<op_t*>(dOt + ltr_off[i]) = doch[i];
-      if (kInlineDelta) {
-        // the LPR threads that share a row are consecutive lanes
-        float acc = dpart[i];
+      for (int k = 0; k < CH; ++k) {
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)och[k][e] * (float)doch[k][e];
 #pragma unroll
         for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-        if ((tid + i * NT) % LPR == 0) Ds[crow[i]] = acc;
+        if (cc0 == 0) Ds[r0 + k * RPI] = acc;
       }
     }
     if (tid < BM) {
-      Ls[tid] = l_stage;
+      Ls[tid] = l_stage * kRcpLn2;                          // bwd_inner_dk_dv.py:185-186
       if (!kInlineDelta) Ds[tid] = d_stage;
     }
   };
@@ -294,6 +283,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   // ---- one (q-head, Q tile) step -----------------------------------------------
   auto compute = [&](auto masked_tag, int g, int e, int stage) {
     constexpr bool masked = decltype(masked_tag)::value;
+    constexpr int G1 = KS * MB, G4 = TS * DB;
     const int hq = hk * group + g;
     const int m0 = (br.lo + e) * BM;
     char* sp = stage_ptr(stage);
@@ -320,7 +310,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     constexpr int kAhead = 2;
     op_t xa[kAhead + 1][MB];
     op_t pb[TS], sb[TS];
-    f32x4 l4[MB][4], d4[MB][4];
+    // row statistics are read four rows at a time, one read ahead of their use
+    f32x4 l4[2], d4[2];
+    auto stat_ptr = [&](const float* base, int q) { return base + 32 * (q / 4) + 8 * (q % 4) + 4 * hi; };
 
     // ---- S = Q K^T ---------------------------------------------------------------
 #pragma unroll
@@ -336,15 +328,23 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
               *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + (k + kAhead) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
+      for (int mb = 0; mb < MB; ++mb) {
         s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kreg[k], k == 0 ? zero16 : s[mb]);
+        // the next tile's global loads ride behind these MFMAs
+        constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
+        const int gidx = k * MB + mb;
+        if (gidx % every == 0) {
+#pragma unroll
+          for (int q = 0; q < (FETCH_PIECES + G1 - 1) / G1; ++q) {
+            const int piece = gidx / every * ((FETCH_PIECES + G1 - 1) / G1) + q;
+            if (piece < FETCH_PIECES) fetch_piece(piece);
+          }
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     // row statistics of the tile's queries and the first dO operands
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) l4[mb][g] = *reinterpret_cast<const f32x4*>(Ls + 32 * mb + 8 * g + 4 * hi);
+    l4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ls, 0));
 #pragma unroll
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
@@ -354,13 +354,14 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     auto p_el = [&](int E) {
       const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
       const int m = m0 + 32 * mb + 8 * g + 4 * hi + r;
+      if (E % 4 == 0 && E + 4 < 16 * MB) l4[(E / 4 + 1) & 1] = *reinterpret_cast<const f32x4*>(stat_ptr(Ls, E / 4 + 1));
       // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
       float x;
       if (kBias) {
         const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
-        x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)mm * a.sb_m] * kLog2e) - l4[mb][g][r];
+        x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)mm * a.sb_m] * kLog2e) - l4[(E / 4) & 1][r];
       } else {
-        x = __builtin_fmaf(s[mb][i], qk_scale, -l4[mb][g][r]);
+        x = __builtin_fmaf(s[mb][i], qk_scale, -l4[(E / 4) & 1][r]);
       }
       if (masked) {
         bool vis = (m < si.seqlen_q) & key_ok;
@@ -388,9 +389,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     };
     auto ds_el = [&](int E) {
       const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
+      if (E % 4 == 0 && E + 4 < 16 * MB) d4[(E / 4 + 1) & 1] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, E / 4 + 1));
       float dpv = dp[mb][i];
       if (kDropout) dpv = keep_bit[E] ? dpv * dst.scale : 0.f;   // :239-240
-      dp[mb][i] = s[mb][i] * (dpv - d4[mb][g][r]);                // ds uses the undropped p (:242)
+      dp[mb][i] = s[mb][i] * (dpv - d4[(E / 4) & 1][r]);          // ds uses the undropped p (:242)
     };
     auto ds_pair = [&](int E) {  // E odd: ds cast to Q's dtype
       sb[E / 8][E % 8 - 1] = Tr::cvt(dp[E / 16][E % 16 - 1]);
@@ -432,10 +434,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       }
     }
     // delta of the tile's queries, first transposed dO operands
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) d4[mb][g] = *reinterpret_cast<const f32x4*>(Ds + 32 * mb + 8 * g + 4 * hi);
+    d4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 0));
     op_t ta[2][DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(dOt + db * 32, TSTR);
@@ -480,13 +479,27 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
           ta[(t + 1) & 1][db] = lds_read_tr8<T>(Qt + (t + 1) * 16 * TSTR + db * 32, TSTR);
       }
 #pragma unroll
-      for (int db = 0; db < DB; ++db) dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
+      for (int db = 0; db < DB; ++db) {
+        dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
+        // the next tile's LDS writes ride behind these MFMAs
+        constexpr int per = (STORE_PIECES + G4 - 1) / G4;
+#pragma unroll
+        for (int q = 0; q < per; ++q) {
+          const int piece = (t * DB + db) * per + q;
+          if (piece < STORE_PIECES) store_piece(piece, stage ^ 1);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
+    store_stats(stage ^ 1);
   };
 
-  load_tile(0, 0);
-  store_tile(0);
+  fetch_begin(true, 0, 0);
+#pragma unroll
+  for (int i = 0; i < FETCH_PIECES; ++i) fetch_piece(i);
+#pragma unroll
+  for (int i = 0; i < STORE_PIECES; ++i) store_piece(i, 0);
+  store_stats(0);
   __syncthreads();
   // Per q-head the Q tiles come as [masked | full | masked]; each run has its own
   // loop so that the loop bodies are straight-line code.
@@ -498,9 +511,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const int stage = it & 1;
     int g_nxt = g_cur, e_nxt = e_cur + 1;
     if (e_nxt == ntq) { e_nxt = 0; ++g_nxt; }
-    if (it + 1 < total) load_tile(g_nxt, e_nxt);
+    fetch_begin(it + 1 < total, g_nxt, e_nxt);
     compute(masked_tag, g_cur, e_cur, stage);
-    if (it + 1 < total) store_tile(stage ^ 1);
     __syncthreads();
     ++it;
     g_cur = g_nxt; e_cur = e_nxt;
