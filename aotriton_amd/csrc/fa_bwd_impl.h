@@ -652,162 +652,210 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     for (int i = 0; i < 16; ++i) dq[db][i] = 0.f;
   const float qk_scale = a.sm_scale * kLog2e;
 
+  // K and V tiles travel global -> registers -> LDS in 16-byte pieces that are issued
+  // between the MFMAs of the running tile (loads behind S^T = K Q^T, LDS writes behind
+  // dQ^T += K^T dS^T).  Buffer loads with a descriptor rebased on every tile: rows past
+  // the end of the sequence read as zero (dS is 0 there), and a descriptor of zero
+  // records turns the fetch after the last tile into a no-op.
+  constexpr int LPR = D / 8;                     // 16-byte pieces per row
+  constexpr int RPI = NT / LPR;                  // rows between two pieces of one thread
+  static_assert((BN * D / 8) % NT == 0 && NT % LPR == 0, "threads must cover the tile evenly");
   op_t kch[CH], vch[CH];
-  int crow[CH];
-  uint32_t koff[CH], voff[CH], lrow_off[CH], ltr_off[CH];
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int idx = tid + i * NT;
-    const int r = idx / (D / 8), cc = idx % (D / 8);
-    crow[i] = r;
-    koff[i] = (uint32_t)(r * (int)a.sk.s + cc * 8);
-    voff[i] = (uint32_t)(r * (int)a.sv.s + cc * 8);
-    lrow_off[i] = (uint32_t)(r * RSTR + cc * 8);
-    ltr_off[i] = (uint32_t)(r * TSTR + cc * 8);
-  }
+  const int r0 = tid / LPR, cc0 = tid % LPR;
+  const int k_voff = r0 * (int)a.sk.s * 2 + cc0 * 16, v_voff = r0 * (int)a.sv.s * 2 + cc0 * 16;
+  const int k_soff = RPI * (int)a.sk.s * 2, v_soff = RPI * (int)a.sv.s * 2;
+  const int lrow0 = r0 * RSTR + cc0 * 8, ltr0 = r0 * TSTR + cc0 * 8;      // elements
   // lane-constant part of the transposing-read address (see lds_read_tr8)
   const int tr_lane = (4 * hi + (lane & 15) / 4) * TSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  auto load_tile = [&](int j) {
-    const T* kt = kbase + (int64_t)j * BN * a.sk.s;
-    const T* vt = vbase + (int64_t)j * BN * a.sv.s;
-    if ((j + 1) * BN <= si.seqlen_k) {
-#pragma unroll
-      for (int i = 0; i < CH; ++i) kch[i] = *reinterpret_cast<const op_t*>(kt + koff[i]);
-#pragma unroll
-      for (int i = 0; i < CH; ++i) vch[i] = *reinterpret_cast<const op_t*>(vt + voff[i]);
-    } else {
-      // ragged last K tile: rows past the end are zero (K: dS is 0 there) / clamped (V)
-      const int nvalid = si.seqlen_k - j * BN;
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const bool ok = crow[i] < nvalid;
-        const int r = ok ? crow[i] : nvalid - 1;
-        const int cc8 = (tid + i * NT) % (D / 8) * 8;
-        op_t x = *reinterpret_cast<const op_t*>(kt + (int64_t)r * a.sk.s + cc8);
-        if (!ok) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = 0;
-        }
-        kch[i] = x;
-        vch[i] = *reinterpret_cast<const op_t*>(vt + (int64_t)r * a.sv.s + cc8);
-      }
-    }
+  const T* kt = kbase + (int64_t)br.lo * BN * a.sk.s;
+  const T* vt = vbase + (int64_t)br.lo * BN * a.sv.s;
+  const int64_t k_step = (int64_t)BN * a.sk.s, v_step = (int64_t)BN * a.sv.s;
+  int rows_left = si.seqlen_k - br.lo * BN;      // > 0
+  __amdgpu_buffer_rsrc_t k_rs, v_rs;
+  // tiles are fetched in ascending order; `live` false: nothing is fetched
+  auto fetch_begin = [&](bool live) {
+    int rows = rows_left < BN ? rows_left : BN;
+    rows = live ? rows : 0;
+    const bool any = rows > 0;
+    k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, any ? ((rows - 1) * (int)a.sk.s + D) * 2 : 0,
+                                             0x00020000);
+    v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, any ? ((rows - 1) * (int)a.sv.s + D) * 2 : 0,
+                                             0x00020000);
+    if (live) { kt += k_step; vt += v_step; rows_left -= BN; }
   };
-  auto store_tile = [&](int stage) {
+  constexpr int FETCH_PIECES = 2 * CH;
+  auto fetch_piece = [&](int i) {        // K pieces first, then V
+    if (i < CH)
+      kch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff, i * k_soff, 0));
+    else
+      vch[i - CH] =
+          __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_voff, (i - CH) * v_soff, 0));
+  };
+  constexpr int STORE_PIECES = 3 * CH;
+  auto store_piece = [&](int i, int stage) {   // K: two copies (row reads, transposing reads); V: one
     T* Ks = reinterpret_cast<T*>(smem_raw + stage * SM::STAGE_BYTES);
     T* Vs = Ks + SM::ROW_ELEMS;
     T* Kt = Vs + SM::ROW_ELEMS;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      *reinterpret_cast<op_t*>(Ks + lrow_off[i]) = kch[i];
-      *reinterpret_cast<op_t*>(Kt + ltr_off[i]) = kch[i];
-      *reinterpret_cast<op_t*>(Vs + lrow_off[i]) = vch[i];
+    if (i < 2 * CH) {
+      const int k = i / 2;
+      T* dst = (i % 2 == 0) ? Ks + lrow0 + k * RPI * RSTR : Kt + ltr0 + k * RPI * TSTR;
+      *reinterpret_cast<op_t*>(dst) = kch[k];
+    } else {
+      const int k = i - 2 * CH;
+      *reinterpret_cast<op_t*>(Vs + lrow0 + k * RPI * RSTR) = vch[k];
     }
   };
 
   auto compute = [&](auto masked_tag, int j, int stage) {
     constexpr bool masked = decltype(masked_tag)::value;
+    constexpr int G1 = KS * MB, G4 = TS * DB;
     const T* Ks = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + c * RSTR + hi * 8;
     const T* Vs = Ks + SM::ROW_ELEMS;
     const T* Kt = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + 2 * SM::ROW_ELEMS + tr_lane;
     f32x16 s[MB], dp[MB];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    op_t xa[2][MB];
-    __builtin_amdgcn_s_setprio(2);
+    // The vector ALU work is spread over MFMAs that do not depend on it: p = exp2(...)
+    // of S runs behind the MFMAs of dP, ds = p (dP - delta) of one 16-key step behind
+    // the dQ MFMAs of the step before.  Fences keep the hand-made order.
+    constexpr int kAhead = 2;
+    op_t xa[kAhead + 1][MB];
+    op_t sb[TS];
+    uint32_t keep[kDropout ? 4 * MB : 1];
+
+    // ---- S^T = K Q^T -------------------------------------------------------------
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR);
+    for (int k = 0; k < kAhead; ++k)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + k * 16);
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
-      if (k + 1 < KS) {
+      if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + (k + 1) * 16);
+          xa[(k + kAhead) % (kAhead + 1)][mb] =
+              *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + (k + kAhead) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) s[mb] = Tr::mfma(xa[k & 1][mb], qreg[k], k == 0 ? zero16 : s[mb]);
+      for (int mb = 0; mb < MB; ++mb) {
+        s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], qreg[k], k == 0 ? zero16 : s[mb]);
+        // the next tile's global loads ride behind these MFMAs
+        constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
+        constexpr int per = (FETCH_PIECES + G1 - 1) / G1;
+        const int gidx = k * MB + mb;
+        if (gidx % every == 0) {
+#pragma unroll
+          for (int q = 0; q < per; ++q) {
+            const int piece = gidx / every * per + q;
+            if (piece < FETCH_PIECES) fetch_piece(piece);
+          }
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xa[0][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR);
+    for (int k = 0; k < kAhead; ++k)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + k * 16);
+
+    // element E = 16*mb + i of the tile: p, kept in s
+    auto p_el = [&](int E) {
+      const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
+      const int n = j * BN + 32 * mb + 8 * g + 4 * hi + r;
+      float x;
+      if (kBias) {
+        const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
+        x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)nn * a.sb_n] * kLog2e) - l_row;
+      } else {
+        x = __builtin_fmaf(s[mb][i], qk_scale, -l_row);
+      }
+      if (masked) {
+        bool vis = n < si.seqlen_k;
+        if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
+        x = vis ? x : -__builtin_inff();
+      }
+      s[mb][i] = fast_exp2(x);
+    };
+    auto ds_el = [&](int E) {
+      const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
+      const int n = j * BN + 32 * mb + 8 * g + 4 * hi + r;
+      if (kDropout && r == 0) keep[E / 4] = dropout_keep4(dst, row, n);
+      float dpv = dp[mb][i];
+      if (kDropout) dpv = ((keep[E / 4] >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
+      const float dsv = s[mb][i] * (dpv - d_row);
+      dp[mb][i] = dsv;
+      if (kBias && dbptr != nullptr && row_ok && n < si.seqlen_k)
+        dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);                            // bwd_inner_dq.py:200-204
+      if (E & 1) {   // ds cast to K's dtype, pair by pair
+        sb[E / 8][E % 8 - 1] = Tr::cvt(dp[mb][i - 1]);
+        sb[E / 8][E % 8] = Tr::cvt(dsv);
+      }
+    };
+
+    // ---- dP^T = V dO^T, with p behind its MFMAs -----------------------------------
+    constexpr int EPG1 = 16 / KS;          // elements per MFMA
+    static_assert(16 % KS == 0, "element split");
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
-      if (k + 1 < KS) {
+      if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + 1) & 1][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + (k + 1) * 16);
+          xa[(k + kAhead) % (kAhead + 1)][mb] =
+              *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + (k + kAhead) * 16);
       }
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) dp[mb] = Tr::mfma(xa[k & 1][mb], doreg[k], k == 0 ? zero16 : dp[mb]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int mb = 0; mb < MB; ++mb) {
+        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], doreg[k], k == 0 ? zero16 : dp[mb]);
+#pragma unroll
+        for (int e = 0; e < EPG1; ++e) p_el((k * MB + mb) * EPG1 + e);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    __builtin_amdgcn_s_setprio(0);
     op_t ta[2][DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Kt + db * 32, TSTR);
-
+    // ds of the first 16-key step has nothing to hide behind
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int nb = j * BN + 32 * mb + 8 * g + 4 * hi;
-        uint32_t keep = 0xF;
-        if (kDropout) keep = dropout_keep4(dst, row, nb);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = 4 * g + r;
-          const int n = nb + r;
-          float x;
-          if (kBias) {
-            const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
-            x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)nn * a.sb_n] * kLog2e) - l_row;
-          } else {
-            x = __builtin_fmaf(s[mb][i], qk_scale, -l_row);
-          }
-          if (masked) {
-            bool vis = n < si.seqlen_k;
-            if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
-            x = vis ? x : -__builtin_inff();
-          }
-          const float p = fast_exp2(x);
-          float dpv = dp[mb][i];
-          if (kDropout) dpv = ((keep >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
-          const float dsv = p * (dpv - d_row);
-          dp[mb][i] = dsv;
-          if (kBias && dbptr != nullptr && row_ok && n < si.seqlen_k)
-            dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);                      // bwd_inner_dq.py:200-204
-        }
-      }
-    op_t sb[TS];
-#pragma unroll
-    for (int t = 0; t < TS; ++t) sb[t] = pack8<T>(dp[t / 2], t % 2);
+    for (int E = 0; E < 8; ++E) ds_el(E);
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(2);
+
+    // ---- dQ^T += K^T dS^T, with the next step's ds and the LDS writes behind its MFMAs ----
+    constexpr int EPG3 = 8 / DB;
+    static_assert(8 % DB == 0, "element split");
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
-      if (t + 1 < TS) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = lds_read_tr8<T>(Kt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+      for (int db = 0; db < DB; ++db) {
+        if (t + 1 < TS) ta[(t + 1) & 1][db] = lds_read_tr8<T>(Kt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+        dq[db] = Tr::mfma(ta[t & 1][db], sb[t], dq[db]);
+        if (t + 1 < TS) {
+#pragma unroll
+          for (int e = 0; e < EPG3; ++e) ds_el(8 * (t + 1) + db * EPG3 + e);
+        }
+        constexpr int per = (STORE_PIECES + G4 - 1) / G4;
+#pragma unroll
+        for (int q = 0; q < per; ++q) {
+          const int piece = (t * DB + db) * per + q;
+          if (piece < STORE_PIECES) store_piece(piece, stage ^ 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int db = 0; db < DB; ++db) dq[db] = Tr::mfma(ta[t & 1][db], sb[t], dq[db]);
-      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_s_setprio(0);
   };
 
-  load_tile(br.lo);
-  store_tile(0);
+  fetch_begin(true);
+#pragma unroll
+  for (int i = 0; i < FETCH_PIECES; ++i) fetch_piece(i);
+#pragma unroll
+  for (int i = 0; i < STORE_PIECES; ++i) store_piece(i, 0);
   __syncthreads();
   // K tiles come as [masked | full | masked]; one straight-line loop per run
   {
     int j = br.lo;
     auto step = [&](auto masked_tag) {
       const int stage = (j - br.lo) & 1;
-      if (j < br.hi) load_tile(j + 1);
+      fetch_begin(j < br.hi);
       compute(masked_tag, j, stage);
-      if (j < br.hi) store_tile(stage ^ 1);
       __syncthreads();
       ++j;
     };
