@@ -63,23 +63,17 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
 // are simply stored twice, once per padding: no register transposes, no bank
 // conflicts on either access pattern.
 template <int D, int BM>
-struct DkDvSmem {   // per stage: Q, dO for row reads; Q, dO for transposing reads; L, delta
-  static constexpr int RSTR = D + 8;
-  static constexpr int TSTR = D + 32;
-  static constexpr int ROW_ELEMS = BM * RSTR;
-  static constexpr int TR_ELEMS = BM * TSTR;
-  static constexpr int STAGE_BYTES = (2 * ROW_ELEMS + 2 * TR_ELEMS) * 2 + 2 * BM * 4;
+struct DkDvSmem {   // per stage: Q, dO (swizzled, one copy each); L, delta
+  static constexpr int TILE_BYTES = BM * D * 2;
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * BM * 4;
   static constexpr int STAGES = 2;
   static constexpr int BYTES = STAGES * STAGE_BYTES;
 };
 
 template <int D, int BN>
-struct DqSmem {     // per stage: K, V for row reads; K for transposing reads
-  static constexpr int RSTR = D + 8;
-  static constexpr int TSTR = D + 32;
-  static constexpr int ROW_ELEMS = BN * RSTR;
-  static constexpr int TR_ELEMS = BN * TSTR;
-  static constexpr int STAGE_BYTES = (2 * ROW_ELEMS + TR_ELEMS) * 2;
+struct DqSmem {     // per stage: K, V (swizzled)
+  static constexpr int TILE_BYTES = BN * D * 2;
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;
   static constexpr int STAGES = 2;
   static constexpr int BYTES = STAGES * STAGE_BYTES;
 };
@@ -102,7 +96,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   constexpr int NT = NW * 64;
   constexpr int BN = NW * 32;
   constexpr int KS = D / 16, MB = BM / 32, DB = D / 32, TS = BM / 16;
-  constexpr int RSTR = SM::RSTR, TSTR = SM::TSTR;
+  constexpr int ROWB = Swz<D>::ROWB;
   constexpr int NCH = BM * D / 8;                // 16-byte chunks per tile, per tensor
   constexpr int CH = (NCH + NT - 1) / NT;        // chunks per thread, per tensor
   constexpr int LPR = D / 8;                     // lanes that share one row
@@ -167,8 +161,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   const int ntq = br.hi - br.lo + 1;
   const int total = group * ntq;
   const float qk_scale = a.sm_scale * kLog2e;
-  // lane-constant part of the transposing-read address (see lds_read_tr8)
-  const int tr_lane = (4 * hi + (lane & 15) / 4) * TSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  // lane constants of the two LDS access patterns
+  const int row_a = Swz<D>::row_base(lane), tr_a0 = Swz<D>::tr_base(lane, 0), tr_a1 = Swz<D>::tr_base(lane, 1);
 
   auto stage_ptr = [&](int stage) { return smem_raw + stage * SM::STAGE_BYTES; };
 
@@ -187,7 +181,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   const int q_voff = r0 * (int)a.sq.s * 2 + cc0 * 16, do_voff = r0 * (int)a.sdo.s * 2 + cc0 * 16,
             o_voff = r0 * (int)a.so.s * 2 + cc0 * 16;                     // bytes inside a tile
   const int q_soff = RPI * (int)a.sq.s * 2, do_soff = RPI * (int)a.sdo.s * 2, o_soff = RPI * (int)a.so.s * 2;
-  const int lrow0 = r0 * RSTR + cc0 * 8, ltr0 = r0 * TSTR + cc0 * 8;      // elements
+  int lds_off[CH];                                                        // bytes inside a tile
+#pragma unroll
+  for (int k = 0; k < CH; ++k) lds_off[k] = Swz<D>::addr(r0 + k * RPI, cc0);
 
   // Tile base pointers advance incrementally (one 64-bit add per tensor and tile);
   // with one wave per SIMD a chain of scalar multiplies per tile is not hidden.
@@ -244,22 +240,15 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         och[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(o_rs, o_voff, k * o_soff, 0));
     }
   };
-  constexpr int STORE_PIECES = 4 * CH;
-  auto store_piece = [&](int i, int stage) {   // same order as the fetches; two copies each
+  constexpr int STORE_PIECES = 2 * CH;
+  auto store_piece = [&](int i, int stage) {   // same order as the fetches
     char* sp = stage_ptr(stage);
-    T* Qs = reinterpret_cast<T*>(sp);
-    T* dOs = Qs + SM::ROW_ELEMS;
-    T* Qt = dOs + SM::ROW_ELEMS;
-    T* dOt = Qt + SM::TR_ELEMS;
-    const int tensor = i / (2 * CH), k = (i % (2 * CH)) / 2, copy = i % 2;
-    const op_t v = tensor == 0 ? qch[k] : doch[k];
-    T* dst = copy == 0 ? (tensor == 0 ? Qs : dOs) + lrow0 + k * RPI * RSTR
-                       : (tensor == 0 ? Qt : dOt) + ltr0 + k * RPI * TSTR;
-    *reinterpret_cast<op_t*>(dst) = v;
+    if (i < CH) *reinterpret_cast<op_t*>(sp + lds_off[i]) = qch[i];
+    else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = doch[i - CH];
   };
   auto store_stats = [&](int stage) {
     char* sp = stage_ptr(stage);
-    float* Ls = reinterpret_cast<float*>(reinterpret_cast<T*>(sp) + 2 * SM::ROW_ELEMS + 2 * SM::TR_ELEMS);
+    float* Ls = reinterpret_cast<float*>(sp + 2 * SM::TILE_BYTES);
     float* Ds = Ls + BM;
     if (kInlineDelta) {
       // delta recomputed from O and dO (bwd_kernel_fuse.py:307-310); the LPR threads
@@ -287,11 +276,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const int hq = hk * group + g;
     const int m0 = (br.lo + e) * BM;
     char* sp = stage_ptr(stage);
-    const T* Qs = reinterpret_cast<const T*>(sp) + c * RSTR + hi * 8;
-    const T* dOs = reinterpret_cast<const T*>(sp) + SM::ROW_ELEMS + c * RSTR + hi * 8;
-    const T* Qt = reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + tr_lane;
-    const T* dOt = Qt + SM::TR_ELEMS;
-    const float* Ls = reinterpret_cast<const float*>(reinterpret_cast<const T*>(sp) + 2 * SM::ROW_ELEMS + 2 * SM::TR_ELEMS);
+    const char* Qb = sp;
+    const char* dOb = sp + SM::TILE_BYTES;
+    const float* Ls = reinterpret_cast<const float*>(sp + 2 * SM::TILE_BYTES);
     const float* Ds = Ls + BM;
 
     f32x16 s[MB], dp[MB];
@@ -318,14 +305,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 #pragma unroll
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + k * 16);
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Qb, row_a, k, mb);
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
       if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] =
-              *reinterpret_cast<const op_t*>(Qs + mb * 32 * RSTR + (k + kAhead) * 16);
+          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Qb, row_a, k + kAhead, mb);
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
@@ -348,7 +334,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 #pragma unroll
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + k * 16);
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(dOb, row_a, k, mb);
 
     // element E = 16*mb + i of the tile: p (kept in s, undropped) and its operand form
     auto p_el = [&](int E) {
@@ -407,8 +393,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] =
-              *reinterpret_cast<const op_t*>(dOs + mb * 32 * RSTR + (k + kAhead) * 16);
+          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(dOb, row_a, k + kAhead, mb);
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
@@ -437,7 +422,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     d4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 0));
     op_t ta[2][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(dOt + db * 32, TSTR);
+    for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, 0, db);
 
     // ---- dV^T += dO^T P, with ds behind its MFMAs --------------------------------
     constexpr int G3 = TS * DB;
@@ -447,7 +432,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     for (int t = 0; t < TS; ++t) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        if (t + 1 < TS) ta[(t + 1) & 1][db] = lds_read_tr8<T>(dOt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+        if (t + 1 < TS) ta[(t + 1) & 1][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, t + 1, db);
         dv[db] = Tr::mfma(ta[t & 1][db], pb[t], dv[db]);
         const int gidx = t * DB + db;
         if (EPG3 >= 1) {
@@ -470,13 +455,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     }
     // ---- dK^T += Q^T dS ----------------------------------------------------------
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Qt + db * 32, TSTR);
+    for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, 0, db);
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       if (t + 1 < TS) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = lds_read_tr8<T>(Qt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+          ta[(t + 1) & 1][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, t + 1, db);
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
@@ -553,7 +538,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   constexpr int NT = NW * 64;
   constexpr int BM = NW * 32;
   constexpr int KS = D / 16, MB = BN / 32, DB = D / 32, TS = BN / 16;
-  constexpr int RSTR = SM::RSTR, TSTR = SM::TSTR;
+  constexpr int ROWB = Swz<D>::ROWB;
   constexpr int CH = (BN * D / 8) / NT;          // 16-byte chunks per thread, per tensor
   static_assert((BN * D / 8) % NT == 0, "tile must split evenly");
 
@@ -664,9 +649,11 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   const int r0 = tid / LPR, cc0 = tid % LPR;
   const int k_voff = r0 * (int)a.sk.s * 2 + cc0 * 16, v_voff = r0 * (int)a.sv.s * 2 + cc0 * 16;
   const int k_soff = RPI * (int)a.sk.s * 2, v_soff = RPI * (int)a.sv.s * 2;
-  const int lrow0 = r0 * RSTR + cc0 * 8, ltr0 = r0 * TSTR + cc0 * 8;      // elements
-  // lane-constant part of the transposing-read address (see lds_read_tr8)
-  const int tr_lane = (4 * hi + (lane & 15) / 4) * TSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  int lds_off[CH];                                                        // bytes inside a tile
+#pragma unroll
+  for (int k = 0; k < CH; ++k) lds_off[k] = Swz<D>::addr(r0 + k * RPI, cc0);
+  // lane constants of the two LDS access patterns
+  const int row_a = Swz<D>::row_base(lane), tr_a0 = Swz<D>::tr_base(lane, 0), tr_a1 = Swz<D>::tr_base(lane, 1);
 
   const T* kt = kbase + (int64_t)br.lo * BN * a.sk.s;
   const T* vt = vbase + (int64_t)br.lo * BN * a.sv.s;
@@ -692,27 +679,18 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       vch[i - CH] =
           __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_voff, (i - CH) * v_soff, 0));
   };
-  constexpr int STORE_PIECES = 3 * CH;
-  auto store_piece = [&](int i, int stage) {   // K: two copies (row reads, transposing reads); V: one
-    T* Ks = reinterpret_cast<T*>(smem_raw + stage * SM::STAGE_BYTES);
-    T* Vs = Ks + SM::ROW_ELEMS;
-    T* Kt = Vs + SM::ROW_ELEMS;
-    if (i < 2 * CH) {
-      const int k = i / 2;
-      T* dst = (i % 2 == 0) ? Ks + lrow0 + k * RPI * RSTR : Kt + ltr0 + k * RPI * TSTR;
-      *reinterpret_cast<op_t*>(dst) = kch[k];
-    } else {
-      const int k = i - 2 * CH;
-      *reinterpret_cast<op_t*>(Vs + lrow0 + k * RPI * RSTR) = vch[k];
-    }
+  constexpr int STORE_PIECES = 2 * CH;
+  auto store_piece = [&](int i, int stage) {   // same order as the fetches
+    char* sp = smem_raw + stage * SM::STAGE_BYTES;
+    if (i < CH) *reinterpret_cast<op_t*>(sp + lds_off[i]) = kch[i];
+    else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = vch[i - CH];
   };
 
   auto compute = [&](auto masked_tag, int j, int stage) {
     constexpr bool masked = decltype(masked_tag)::value;
     constexpr int G1 = KS * MB, G4 = TS * DB;
-    const T* Ks = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + c * RSTR + hi * 8;
-    const T* Vs = Ks + SM::ROW_ELEMS;
-    const T* Kt = reinterpret_cast<const T*>(smem_raw + stage * SM::STAGE_BYTES) + 2 * SM::ROW_ELEMS + tr_lane;
+    const char* Kb = smem_raw + stage * SM::STAGE_BYTES;
+    const char* Vb = Kb + SM::TILE_BYTES;
     f32x16 s[MB], dp[MB];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // The vector ALU work is spread over MFMAs that do not depend on it: p = exp2(...)
@@ -727,14 +705,13 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 #pragma unroll
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + k * 16);
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Kb, row_a, k, mb);
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
       if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] =
-              *reinterpret_cast<const op_t*>(Ks + mb * 32 * RSTR + (k + kAhead) * 16);
+          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Kb, row_a, k + kAhead, mb);
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
@@ -756,7 +733,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 #pragma unroll
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + k * 16);
+      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Vb, row_a, k, mb);
 
     // element E = 16*mb + i of the tile: p, kept in s
     auto p_el = [&](int E) {
@@ -800,8 +777,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] =
-              *reinterpret_cast<const op_t*>(Vs + mb * 32 * RSTR + (k + kAhead) * 16);
+          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Vb, row_a, k + kAhead, mb);
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
@@ -813,7 +789,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     }
     op_t ta[2][DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = lds_read_tr8<T>(Kt + db * 32, TSTR);
+    for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(Kb, tr_a0, tr_a1, 0, db);
     // ds of the first 16-key step has nothing to hide behind
 #pragma unroll
     for (int E = 0; E < 8; ++E) ds_el(E);
@@ -826,7 +802,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     for (int t = 0; t < TS; ++t) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        if (t + 1 < TS) ta[(t + 1) & 1][db] = lds_read_tr8<T>(Kt + (t + 1) * 16 * TSTR + db * 32, TSTR);
+        if (t + 1 < TS) ta[(t + 1) & 1][db] = swz_read_tr<T, D>(Kb, tr_a0, tr_a1, t + 1, db);
         dq[db] = Tr::mfma(ta[t & 1][db], sb[t], dq[db]);
         if (t + 1 < TS) {
 #pragma unroll

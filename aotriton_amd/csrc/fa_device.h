@@ -98,6 +98,47 @@ __device__ __forceinline__ typename Traits<T>::op_t lds_read_tr8(const T* p, int
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Swizzled LDS tile of rows of D 16-bit elements, no padding.  The 16-byte chunk `ch`
+// of row r lives at chunk position ch ^ f(r) of that row.  f is chosen so that both
+// access patterns of the kernels sweep all 64 banks once: the 16-byte row reads of an
+// MFMA operand (16 consecutive rows, same chunk) and the transposing reads (4
+// consecutive rows x 4 consecutive chunks per half-wave).  A tile can therefore
+// serve both as the row operand of one GEMM and as the transposed operand of another.
+template <int D>
+struct Swz {
+  static constexpr int ROWB = D * 2;
+  static __device__ __forceinline__ int f(int r) {
+    return D == 64 ? ((((r >> 1) & 1) << 2) | ((r >> 2) & 3)) : (((r & 3) << 2) | ((r >> 2) & 3));
+  }
+  // byte offset of chunk ch of row r
+  static __device__ __forceinline__ int addr(int r, int ch) { return r * ROWB + ((ch ^ f(r)) << 4); }
+  // lane constant of the row reads: MFMA operand row = lane%32 (+32*mb), k-slots 8*hi..
+  static __device__ __forceinline__ int row_base(int lane) { return addr(lane & 31, lane >> 5); }
+  // lane constants of the transposing reads (rows 8*w + 4*hi + (lane%16)/4 of a 16-row step)
+  static __device__ __forceinline__ int tr_base(int lane, int w) {
+    const int r = 8 * w + 4 * (lane >> 5) + (lane & 15) / 4;
+    const int ch = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    return addr(r, ch) + 8 * (lane & 1);
+  }
+};
+// row operand of k-step k, 32-row block mb (f depends on r % 16 only, so the block is a
+// plain offset and the k-step flips chunk bits)
+template <typename T, int D>
+__device__ __forceinline__ typename Traits<T>::op_t swz_read_row(const char* tile, int row_base, int k, int mb) {
+  return *reinterpret_cast<const typename Traits<T>::op_t*>(tile + ((row_base ^ (k << 5)) + mb * 32 * Swz<D>::ROWB));
+}
+// transposed operand: k-slots are rows 16*t + 8*w + 4*hi + j of the tile, M/N index is
+// column 32*db + lane%32 (see lds_read_tr8 for the hardware's lane mapping)
+template <typename T, int D>
+__device__ __forceinline__ typename Traits<T>::op_t swz_read_tr(const char* tile, int tr_base0, int tr_base1,
+                                                                int t, int db) {
+  const typename Traits<T>::q4_t lo = Traits<T>::lds_read_tr(
+      reinterpret_cast<const T*>(tile + ((tr_base0 ^ (db << 6)) + t * 16 * Swz<D>::ROWB)));
+  const typename Traits<T>::q4_t hi = Traits<T>::lds_read_tr(
+      reinterpret_cast<const T*>(tile + ((tr_base1 ^ (db << 6)) + t * 16 * Swz<D>::ROWB)));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // Sum of the 8 (already rounded) elements of an operand, added to acc.
 template <typename T>
 __device__ __forceinline__ float sum8(typename Traits<T>::op_t v, float acc) {
