@@ -270,7 +270,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   };
 
   // ---- one (q-head, Q tile) step -----------------------------------------------
-  auto compute = [&](auto masked_tag, int g, int e, int stage) {
+  auto compute = [&](auto masked_tag, int g, int e, int stage, bool live, int g_nxt, int e_nxt) {
     constexpr bool masked = decltype(masked_tag)::value;
     constexpr int G1 = KS * MB, G4 = TS * DB;
     const int hq = hk * group + g;
@@ -316,10 +316,11 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kreg[k], k == 0 ? zero16 : s[mb]);
-        // the next tile's global loads ride behind these MFMAs
+        // the next tile's descriptors and global loads ride behind these MFMAs
         constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
         const int gidx = k * MB + mb;
-        if (gidx % every == 0) {
+        if (gidx == 0) fetch_begin(live, g_nxt, e_nxt);
+        if (gidx % every == every - 1) {
 #pragma unroll
           for (int q = 0; q < (FETCH_PIECES + G1 - 1) / G1; ++q) {
             const int piece = gidx / every * ((FETCH_PIECES + G1 - 1) / G1) + q;
@@ -496,8 +497,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const int stage = it & 1;
     int g_nxt = g_cur, e_nxt = e_cur + 1;
     if (e_nxt == ntq) { e_nxt = 0; ++g_nxt; }
-    fetch_begin(it + 1 < total, g_nxt, e_nxt);
-    compute(masked_tag, g_cur, e_cur, stage);
+    compute(masked_tag, g_cur, e_cur, stage, it + 1 < total, g_nxt, e_nxt);
     __syncthreads();
     ++it;
     g_cur = g_nxt; e_cur = e_nxt;
@@ -686,7 +686,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = vch[i - CH];
   };
 
-  auto compute = [&](auto masked_tag, int j, int stage) {
+  auto compute = [&](auto masked_tag, int j, int stage, bool live) {
     constexpr bool masked = decltype(masked_tag)::value;
     constexpr int G1 = KS * MB, G4 = TS * DB;
     const char* Kb = smem_raw + stage * SM::STAGE_BYTES;
@@ -716,11 +716,12 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], qreg[k], k == 0 ? zero16 : s[mb]);
-        // the next tile's global loads ride behind these MFMAs
+        // the next tile's descriptors and global loads ride behind these MFMAs
         constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
         constexpr int per = (FETCH_PIECES + G1 - 1) / G1;
         const int gidx = k * MB + mb;
-        if (gidx % every == 0) {
+        if (gidx == 0) fetch_begin(live);
+        if (gidx % every == every - 1) {
 #pragma unroll
           for (int q = 0; q < per; ++q) {
             const int piece = gidx / every * per + q;
@@ -830,8 +831,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     int j = br.lo;
     auto step = [&](auto masked_tag) {
       const int stage = (j - br.lo) & 1;
-      fetch_begin(j < br.hi);
-      compute(masked_tag, j, stage);
+      compute(masked_tag, j, stage, j < br.hi);
       __syncthreads();
       ++j;
     };
