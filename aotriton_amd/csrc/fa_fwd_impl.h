@@ -212,13 +212,8 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     __builtin_amdgcn_s_setprio(0);
   };
 
-  auto sv = [&](int j, int stage, bool masked) {
-    const T* vs = Vs + stage * SM::V_ELEMS + v_lane;
-    // first V^T operands: in flight while the softmax runs
-    op_t va[2][DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db) va[0][db] = lds_read_tr8<T>(vs + db * 32, VSTR);
-
+  // scale, bias and mask on the raw scores
+  auto prepare = [&](int j, bool masked) {
     if (prescale) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -246,45 +241,12 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
           s[mb][i] = vis ? s[mb][i] : -__builtin_inff();
         }
     }
-    float mx = s[0][0];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
-    mx = cross_max(mx);
-    // Lazy rescaling: a row adopts the new maximum only when it grew by more than
-    // 2^8 in the exponent domain; until then p may exceed 1 (at most 256), which
-    // fp32 accumulation and the 16-bit P operand absorb, and the final O = acc / l
-    // is unchanged because l is accumulated against the same reference.
-    const float m_cand = fmaxf(m_i, mx);
-    const bool upd = (m_cand - m_i) * sc > 8.0f;
-    const float m_new = upd ? m_cand : m_i;
-    const float alpha = fast_exp2((m_i - m_new) * sc);
-    const float msc = m_new * sc;
-    m_i = m_new;
+  };
 
+  // dropout, operand conversion and O^T += V^T P^T on the p's held in s
+  op_t va[2][DB];
+  auto finish = [&](int j, const T* vs) {
     op_t pb[TS];
-    float rs = 0.f;
-    // exp2(s*c - m*c) as one fma is exact enough while |m*c| is small; for huge
-    // scores the rounding of m*c alone would be amplified by exp2, so the
-    // difference is formed first (the trap documented at fwd_kernel_inner.py:197-205).
-    const bool big = __builtin_amdgcn_ballot_w64(!(__builtin_fabsf(msc) < 1024.f)) != 0;
-    if (big) {
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[mb][i] = fast_exp2((s[mb][i] - m_new) * sc);
-    } else {
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[mb][i] = fast_exp2(__builtin_fmaf(s[mb][i], sc, -msc));
-    }
-    // the row sum is over the fp32, undropped p (fwd_kernel_inner.py:213-214)
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) rs += s[mb][i];
     if (kDropout) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -298,14 +260,6 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     // P is cast to V's dtype for the second GEMM (:274)
 #pragma unroll
     for (int t = 0; t < TS; ++t) pb[t] = pack8<T>(s[t / 2], t % 2);
-    l_i = l_i * alpha + rs;
-    // rescale the accumulator only when some row of this wave moved its max
-    if (__builtin_amdgcn_ballot_w64(upd) != 0) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-    }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -322,6 +276,93 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     __builtin_amdgcn_s_setprio(0);
   };
 
+  // Speculative softmax step: the exponentials are taken against the reference
+  // maximum the rows already have, with no row maximum of the new tile.  p may
+  // exceed 1 where a row's maximum grew; that is harmless (the final O = acc / l does
+  // not depend on the reference) until the values leave the comfortable range of the
+  // 16-bit P operand, which the row sum reveals.  Returns false, leaving the state
+  // untouched, when some row needs a new reference; the caller then recomputes S and
+  // takes the full step.
+  bool have_ref = false;     // every row of the wave has a usable reference maximum
+  float msc_ref = 0.f;       // m_i * sc
+  auto sv_fast = [&](int j, int stage, bool masked) -> bool {
+    const T* vs = Vs + stage * SM::V_ELEMS + v_lane;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[0][db] = lds_read_tr8<T>(vs + db * 32, VSTR);
+    prepare(j, masked);
+    float rs = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[mb][i] = fast_exp2(__builtin_fmaf(s[mb][i], sc, -msc_ref));
+        rs += s[mb][i];      // the row sum is over the fp32, undropped p (fwd_kernel_inner.py:213-214)
+      }
+    // also catches inf and NaN
+    if (__builtin_amdgcn_ballot_w64(!(rs < 4096.f)) != 0) return false;
+    l_i += rs;
+    finish(j, vs);
+    return true;
+  };
+
+  // full online-softmax step with the row maximum of the tile
+  auto sv = [&](int j, int stage, bool masked) {
+    const T* vs = Vs + stage * SM::V_ELEMS + v_lane;
+    // first V^T operands: in flight while the softmax runs
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[0][db] = lds_read_tr8<T>(vs + db * 32, VSTR);
+    prepare(j, masked);
+    float mx = s[0][0];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
+    mx = cross_max(mx);
+    // Lazy rescaling: a row adopts the new maximum only when it grew by more than
+    // 2^8 in the exponent domain; until then p may exceed 1 (at most 256), which
+    // fp32 accumulation and the 16-bit P operand absorb, and the final O = acc / l
+    // is unchanged because l is accumulated against the same reference.
+    const float m_cand = fmaxf(m_i, mx);
+    const bool upd = (m_cand - m_i) * sc > 8.0f;
+    const float m_new = upd ? m_cand : m_i;
+    const float alpha = fast_exp2((m_i - m_new) * sc);
+    const float msc = m_new * sc;
+    m_i = m_new;
+    msc_ref = msc;
+
+    float rs = 0.f;
+    // exp2(s*c - m*c) as one fma is exact enough while |m*c| is small; for huge
+    // scores the rounding of m*c alone would be amplified by exp2, so the
+    // difference is formed first (the trap documented at fwd_kernel_inner.py:197-205).
+    const bool big = __builtin_amdgcn_ballot_w64(!(__builtin_fabsf(msc) < 1024.f)) != 0;
+    have_ref = !big;         // rows without a visible key so far keep the seed: they fail the fast test
+    if (big) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[mb][i] = fast_exp2((s[mb][i] - m_new) * sc);
+    } else {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[mb][i] = fast_exp2(__builtin_fmaf(s[mb][i], sc, -msc));
+    }
+    // the row sum is over the fp32, undropped p (fwd_kernel_inner.py:213-214)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) rs += s[mb][i];
+    l_i = l_i * alpha + rs;
+    // rescale the accumulator only when some row of this wave moved its max
+    if (__builtin_amdgcn_ballot_w64(upd) != 0) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
+    finish(j, vs);
+  };
+
   // ---- main loop: LDS double buffer, one barrier per tile ---------------------
   load_next_tile();
   store_tile(0);
@@ -331,7 +372,11 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     if (j < br.hi) load_next_tile();
     if (j <= wave_hi) {
       qk(stage);
-      sv(j, stage, !br.is_full(j));
+      const bool masked = !br.is_full(j);
+      if (!(have_ref && sv_fast(j, stage, masked))) {
+        if (have_ref) qk(stage);      // the speculative step consumed S
+        sv(j, stage, masked);
+      }
     }
     if (j < br.hi) store_tile(stage ^ 1);
     __syncthreads();
