@@ -56,12 +56,10 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
 // ---------------------------------------------------------------------------
 // Shared-memory plans
 // ---------------------------------------------------------------------------
-// Every staged tile is row-major.  A tile that is read as rows (16-byte reads, the
-// contraction runs over the head dim) gets rows padded by 16 B; a tile that is read
-// through the transposing LDS loads (the contraction runs over its rows) gets rows
-// padded by 64 B.  Q and dO (dK/dV item) and K (dQ item) are needed both ways and
-// are simply stored twice, once per padding: no register transposes, no bank
-// conflicts on either access pattern.
+// Every staged tile is row-major, unpadded and swizzled (Swz in fa_device.h): the same
+// copy serves the 16-byte row reads of the GEMMs that contract over the head dim and
+// the transposing reads of the GEMMs that contract over the tile's rows, both free
+// of bank conflicts.  Q and dO (dK/dV item) and K (dQ item) are read both ways.
 template <int D, int BM>
 struct DkDvSmem {   // per stage: Q, dO (swizzled, one copy each); L, delta
   static constexpr int TILE_BYTES = BM * D * 2;

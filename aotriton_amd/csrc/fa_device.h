@@ -8,7 +8,8 @@
 // The contraction index is a dummy, so any permutation of k that is applied to
 // both operands is legal.  All kernels exploit that: an accumulator block is
 // re-used as an operand with k-slot (t, hi, j) <-> row 16*t + 8*(j/4) + 4*hi + (j%4),
-// and the other operand is stored in LDS in exactly that order.
+// and the other operand is fetched from a row-major LDS tile with transposing reads
+// that deliver exactly that order.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -49,10 +50,6 @@ template <> struct Traits<bf16_t> {
   static __device__ __forceinline__ q4_t lds_read_tr(const bf16_t* p) {
     return __builtin_bit_cast(q4_t, lds_read_tr_raw(p));
   }
-  static __device__ __forceinline__ float dot2_ones(p2_t a, float acc) {
-    const p2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(a, ones, acc, false);
-  }
   static __device__ __forceinline__ f32x16 mfma(op_t a, op_t b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -65,10 +62,6 @@ template <> struct Traits<f16_t> {
   using p2_t = vec<_Float16, 2>;
   static __device__ __forceinline__ q4_t lds_read_tr(const f16_t* p) {
     return __builtin_bit_cast(q4_t, lds_read_tr_raw(p));
-  }
-  static __device__ __forceinline__ float dot2_ones(p2_t a, float acc) {
-    const p2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
-    return __builtin_amdgcn_fdot2(a, ones, acc, false);
   }
   static __device__ __forceinline__ f32x16 mfma(op_t a, op_t b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
@@ -137,33 +130,6 @@ __device__ __forceinline__ typename Traits<T>::op_t swz_read_tr(const char* tile
   const typename Traits<T>::q4_t hi = Traits<T>::lds_read_tr(
       reinterpret_cast<const T*>(tile + ((tr_base1 ^ (db << 6)) + t * 16 * Swz<D>::ROWB)));
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-// Sum of the 8 (already rounded) elements of an operand, added to acc.
-template <typename T>
-__device__ __forceinline__ float sum8(typename Traits<T>::op_t v, float acc) {
-  using p2_t = typename Traits<T>::p2_t;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const p2_t pr = {v[2 * i], v[2 * i + 1]};
-    acc = Traits<T>::dot2_ones(pr, acc);
-  }
-  return acc;
-}
-
-// acc *= f for an MFMA accumulator that should stay in the accumulator register
-// file: the values are moved out, scaled and moved back explicitly so that the
-// compiler never needs a vector-ALU home for the whole block.
-__device__ __forceinline__ void scale_acc(f32x16& acc, float f) {
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    float t;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(acc[i]));
-    t *= f;
-    float r;
-    asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(r) : "v"(t));
-    acc[i] = r;
-  }
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -296,13 +262,6 @@ __device__ __forceinline__ int xcd_remap_head(int x, int num_heads) {
   constexpr int kXcds = 8;
   if (num_heads % kXcds != 0) return x;
   return (x % kXcds) * (num_heads / kXcds) + x / kXcds;
-}
-
-// LDS position of key `kk` (0..BN-1) inside a transposed tile row: swaps bits 2
-// and 3 of the key index so that one 16-byte read yields the k-slot order
-// described at the top of this file.
-__device__ __forceinline__ int tr_pos(int kk) {
-  return (kk & ~12) | ((kk & 4) << 1) | ((kk & 8) >> 1);
 }
 
 }  // namespace fa

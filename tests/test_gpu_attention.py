@@ -94,3 +94,35 @@ def test_window_bias_dropout_small_config5():
 def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
     # rows with no visible key: O = 0, LSE = +inf, gradients finite
     _run_case(2, 2, 2, 300, 140, 128, torch.bfloat16, causal)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('causal', [False, True])
+def test_row_maximum_grows_along_keys(dtype, causal):
+    # The score scale grows ~40x from the first to the last key, so every row's maximum
+    # is overtaken again and again by later K tiles: a forward that reuses the maximum
+    # of earlier tiles has to notice and renormalise.  Checked against the oracle.
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    B, H, S, D = 1, 2, 1024, 128
+    q, k, v, _, do = make_inputs(B, H, H, S, S, D, dtype, DEV, seed=7)
+    ramp = torch.linspace(0.25, 10.0, S, device=DEV).view(1, 1, S, 1)
+    k = (k.float() * ramp).to(dtype)
+    sm_scale = 1.0 / math.sqrt(D)
+    ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    o, _, L = attention(qg, kg, vg, None, causal, sm_scale, 0.0, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    assert flash.hipGetLastError() == flash.hipError_t.hipSuccess
+    ct, wl, wr = flash.translate_causal(causal)
+    ro, rl, _ = fa_ref.attn_fwd_ref(q.float(), k.float(), v.float(), None, sm_scale, ct, wl, wr, 0.0, None)
+    lo, ll, _ = fa_ref.attn_fwd_ref(q, k, v, None, sm_scale, ct, wl, wr, 0.0, None)
+    check('out', o, ro, lo, FUDGE['out'])
+    assert (L.view(B, H, S) - rl).abs().max().item() <= LSE_ATOL * max(1.0, rl.abs().max().item() / 8)
+    rg = fa_ref.attn_bwd_ref(q.float(), k.float(), v.float(), None, sm_scale, ro, do.float(), rl, ct, wl, wr, 0.0, None)
+    lg = fa_ref.attn_bwd_ref(q, k, v, None, sm_scale, lo, do, ll.to(dtype).float().to(dtype), ct, wl, wr, 0.0, None)
+    check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
+    check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
+    check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
