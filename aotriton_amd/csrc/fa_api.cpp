@@ -354,13 +354,20 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
   const int mt = (s.max_sq + t.block_m - 1) / t.block_m, nt = (s.max_sk + t.block_n - 1) / t.block_n;
+  // 1-D grids of the main kernels: 8 XCDs x (heads per XCD, rounded up to whole groups) x items per head
+  auto grid1d = [&](int heads, int zg, int items) {
+    const int per_xcd = (nz * heads + fa::kNumXcd - 1) / fa::kNumXcd;
+    return fa::kNumXcd * ((per_xcd + zg - 1) / zg) * zg * items;
+  };
+  const int ratio = s.hq / s.hk;
+  out->grid[1] = 1;
+  out->grid[2] = 1;
   switch (kernel_slot) {
-    case 0: out->grid[0] = mt; out->grid[1] = s.hq; break;
-    case 1: out->grid[0] = s.hk; out->grid[1] = nt; break;
-    case 2: out->grid[0] = s.hq; out->grid[1] = mt; break;
-    default: out->grid[0] = s.hk; out->grid[1] = nt + mt * (s.hq / s.hk); break;
+    case 0: out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz; break;
+    case 1: out->grid[0] = grid1d(s.hk, 2, nt); break;
+    case 2: out->grid[0] = grid1d(s.hq, ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2, mt); break;
+    default: out->grid[0] = grid1d(s.hk, 2, nt + mt * ratio); break;
   }
-  out->grid[2] = nz;
   out->backend_index = be;
   out->head_dim = s.d;
   out->flags = (s.windowed ? 1 : 0) | (s.bias ? 2 : 0) | (s.dropout ? 4 : 0) | (s.num_seqlens != 0 ? 8 : 0);

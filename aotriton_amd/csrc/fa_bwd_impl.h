@@ -889,22 +889,32 @@ void bwd_dq_kernel(const BwdArgs a) {
   dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, zh % a.hq, mt, zh / a.hq, smem_raw);
 }
 
-// grid.y = num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
-// (modules/flash/csrc/attn_bwd_fused.cc:13-22, bwd_kernel_fuse.py:107-118).
+// Per (batch, kv-head): num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
+// (modules/flash/csrc/attn_bwd_fused.cc:13-22, bwd_kernel_fuse.py:107-118), laid out on
+// the same 1-D grid as the split kernels: each XCD owns a contiguous range of (batch,
+// kv-head) pairs and walks them in pairs, so the tensors of the heads in flight stay in
+// that XCD's L2.
 template <typename T, int D, int NW, int BM, int BN, bool kWindowed, bool kBias, bool kDropout>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_fused_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  const int hk = xcd_remap_head(blockIdx.x, a.hk);
-  const int item = blockIdx.y;
+  const int group = a.hq / a.hk;
+  const int items = a.num_n_tiles + a.num_m_tiles * group;
+  const int xcd = blockIdx.x % kNumXcd, li = blockIdx.x / kNumXcd;
+  const int per_group = a.zh_group * items;
+  const int gi = li / per_group, gr = li % per_group;
+  const int zl = gi * a.zh_group + gr % a.zh_group;
+  const int zh = xcd * a.zh_per_xcd + zl;
+  if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
+  const int hk = zh % a.hk, z = zh / a.hk;
+  const int item = gr / a.zh_group;
   if (item < a.num_n_tiles) {
-    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true>(a, hk, item, blockIdx.z, smem_raw);
+    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true>(a, hk, item, z, smem_raw);
   } else {
     const int t = item - a.num_n_tiles;
-    const int group = a.hq / a.hk;
     const int h = hk * group + t / a.num_m_tiles;
     const int mt = a.num_m_tiles - 1 - t % a.num_m_tiles;
-    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true>(a, h, mt, blockIdx.z, smem_raw);
+    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true>(a, h, mt, z, smem_raw);
   }
 }
 
@@ -981,7 +991,11 @@ hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dr
   BwdArgs a = a0;
   a.num_n_tiles = (a.seq.max_seqlen_k + NW * 32 - 1) / (NW * 32);
   a.num_m_tiles = (a.seq.max_seqlen_q + NW * 32 - 1) / (NW * 32);
-  dim3 grid(a.hk, a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk), bwd_nseq(a));
+  a.num_zh = bwd_nseq(a) * a.hk;
+  a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
+  a.zh_group = 2;
+  const int items = a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk);
+  dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * items));
 #define FA_CALL(W, B, P) launch_with_lds(bwd_fused_kernel<T, D, NW, BM, BN, W, B, P>, grid, NW * 64, smem, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL

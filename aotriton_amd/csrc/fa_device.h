@@ -255,13 +255,4 @@ __device__ __forceinline__ int64_t lse_offset(const SeqInfo& si, int h, int hq) 
   return ((int64_t)si.batch_index * hq + h) * si.lse_stride + si.q_start;
 }
 
-// Heads are placed on grid.x.  Consecutive workgroup ids round-robin over the 8
-// XCDs, so remap x so that each XCD owns a contiguous range of heads and all
-// tiles of one head (and of one GQA group) share an L2.
-__device__ __forceinline__ int xcd_remap_head(int x, int num_heads) {
-  constexpr int kXcds = 8;
-  if (num_heads % kXcds != 0) return x;
-  return (x % kXcds) * (num_heads / kXcds) + x / kXcds;
-}
-
 }  // namespace fa
