@@ -28,7 +28,7 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16/fp16 MFMA: 256 CU x 2.4 GHz x
 # HBM bytes per launch at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # runs scaled by a 256 MiB elementwise probe (summaries and commands: profiles/*.txt).
 # Counters cannot be read from inside this process, so the figures are recorded here.
-HBM_BYTES_PER_LAUNCH = {'fwd_kernel': 6.3881e8, 'bwd_dkdv_kernel': 1.2514e9, 'bwd_dq_kernel': 1.0490e9}
+HBM_BYTES_PER_LAUNCH = {'fwd_kernel': 6.6010e8, 'bwd_dkdv_kernel': 8.3390e8, 'bwd_dq_kernel': 7.9411e8}
 
 
 def cpu_baseline(B, H, S, D, causal, seed):
@@ -46,8 +46,10 @@ def cpu_baseline(B, H, S, D, causal, seed):
     do = torch.randn(1, h_s, S, D, generator=g)
     ct, wl, wr = (3, -2147483647, -2147483647) if causal else (0, 0, 0)
     sm = 1.0 / math.sqrt(D)
-    fa_ref.sdpa_math_ref(q, k, v, None, sm, ct, wl, wr).backward(do)   # warm-up
-    reps = 4
+    t0 = time.perf_counter()
+    fa_ref.sdpa_math_ref(q, k, v, None, sm, ct, wl, wr).backward(do)   # warm-up, also sizes the sample
+    once = time.perf_counter() - t0
+    reps = max(4, min(64, int(math.ceil(12.0 / max(once, 1e-3)))))     # about 12 s of CPU work
     t0 = time.perf_counter()
     for _ in range(reps):
         q.grad = k.grad = v.grad = None
