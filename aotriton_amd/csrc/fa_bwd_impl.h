@@ -871,7 +871,9 @@ void bwd_dkdv_kernel(const BwdArgs a) {
   const int zl = gi * a.zh_group + gr % a.zh_group;
   const int zh = xcd * a.zh_per_xcd + zl;
   if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
-  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false>(a, zh % a.hk, gr / a.zh_group, zh / a.hk, smem_raw);
+  int z, hk;
+  split_zh(zh, a.num_zh / a.hk, 1, z, hk);
+  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false>(a, hk, gr / a.zh_group, z, smem_raw);
 }
 
 template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
@@ -886,7 +888,9 @@ void bwd_dq_kernel(const BwdArgs a) {
   const int zh = xcd * a.zh_per_xcd + zl;
   if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
   const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
-  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, zh % a.hq, mt, zh / a.hq, smem_raw);
+  int z, h;
+  split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
+  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, h, mt, z, smem_raw);
 }
 
 // Per (batch, kv-head): num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
@@ -906,7 +910,8 @@ void bwd_fused_kernel(const BwdArgs a) {
   const int zl = gi * a.zh_group + gr % a.zh_group;
   const int zh = xcd * a.zh_per_xcd + zl;
   if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
-  const int hk = zh % a.hk, z = zh / a.hk;
+  int z, hk;
+  split_zh(zh, a.num_zh / a.hk, 1, z, hk);
   const int item = gr / a.zh_group;
   if (item < a.num_n_tiles) {
     dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true>(a, hk, item, z, smem_raw);

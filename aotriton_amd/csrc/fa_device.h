@@ -250,6 +250,18 @@ __device__ __forceinline__ SeqInfo get_seq(const SeqArgs& s, int z) {
   return r;
 }
 
+// (sequence, head) of the linear work index zh.  The heads of one GQA group are
+// adjacent, then come the sequences, then the kv-heads: the contiguous range of zh
+// that an XCD owns then holds whole kv-heads across ALL sequences, so XCDs get equal
+// work even when the sequences of a varlen batch differ in length, and neighbours in
+// zh share K/V.  `group` = q-heads per kv-head when zh counts q-heads, 1 when it counts
+// kv-heads.
+__device__ __forceinline__ void split_zh(int zh, int nseq, int group, int& z, int& h) {
+  const int g = zh % group, t = zh / group;
+  z = t % nseq;
+  h = (t / nseq) * group + g;
+}
+
 // _lse_offset, modules/flash/kernel/fwd_kernel_inner.py:38-43
 __device__ __forceinline__ int64_t lse_offset(const SeqInfo& si, int h, int hq) {
   return ((int64_t)si.batch_index * hq + h) * si.lse_stride + si.q_start;

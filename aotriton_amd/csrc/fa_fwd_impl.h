@@ -436,7 +436,9 @@ void fwd_kernel(const FwdArgs a) {
     const int zh = xcd * a.zh_per_xcd + zh_local;
     if (zh_local >= a.zh_per_xcd || zh >= a.num_zh) continue;
     const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
-    fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout>(a, zh / a.hq, zh % a.hq, mt, smem_raw);
+    int z, h;
+    split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
+    fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout>(a, z, h, mt, smem_raw);
   }
 }
 
