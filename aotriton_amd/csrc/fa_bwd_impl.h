@@ -625,6 +625,11 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   if (kBias)
     bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)h * a.sb_h +
            (int64_t)row_c * a.sb_m;
+  // 8-byte bias loads / dB stores need unit column stride and 8-byte aligned rows
+  const bool bias_vec = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 3) == 0 &&
+                        (reinterpret_cast<uintptr_t>(a.bias) & 7) == 0;
+  const bool db_vec = kBias && a.sdb_n == 1 && ((a.sdb_m | a.sdb_h | a.sdb_z) & 3) == 0 &&
+                      (reinterpret_cast<uintptr_t>(a.db) & 7) == 0;
   DropoutState dst{};
   if (kDropout) dst = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
 
@@ -698,6 +703,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     op_t xa[kAhead + 1][MB];
     op_t sb[TS];
     uint32_t keep[kDropout ? 4 * MB : 1];
+    q4_t bias4[2];
+    const bool tile_vec = bias_vec && (j + 1) * BN <= si.seqlen_k;   // the whole tile is inside the row
 
     // ---- S^T = K Q^T -------------------------------------------------------------
 #pragma unroll
@@ -740,8 +747,15 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       const int n = j * BN + 32 * mb + 8 * g + 4 * hi + r;
       float x;
       if (kBias) {
-        const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
-        x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)nn * a.sb_n] * kLog2e) - l_row;
+        float bv;
+        if (tile_vec) {
+          if (r == 0) bias4[(E / 4) & 1] = *reinterpret_cast<const q4_t*>(bptr + n);
+          bv = (float)bias4[(E / 4) & 1][r];
+        } else {
+          const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
+          bv = (float)bptr[(int64_t)nn * a.sb_n];
+        }
+        x = __builtin_fmaf(s[mb][i], qk_scale, bv * kLog2e) - l_row;
       } else {
         x = __builtin_fmaf(s[mb][i], qk_scale, -l_row);
       }
@@ -760,8 +774,18 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       if (kDropout) dpv = ((keep[E / 4] >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
       const float dsv = s[mb][i] * (dpv - d_row);
       dp[mb][i] = dsv;
-      if (kBias && dbptr != nullptr && row_ok && n < si.seqlen_k)
-        dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);                            // bwd_inner_dq.py:200-204
+      if (kBias && dbptr != nullptr && row_ok) {                                 // bwd_inner_dq.py:200-204
+        if (tile_vec && db_vec) {
+          if (r == 3) {
+            q4_t d4v;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) d4v[q] = Tr::cvt(dp[mb][i - 3 + q]);
+            *reinterpret_cast<q4_t*>(dbptr + n - 3) = d4v;
+          }
+        } else if (n < si.seqlen_k) {
+          dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);
+        }
+      }
       if (E & 1) {   // ds cast to K's dtype, pair by pair
         sb[E / 8][E % 8 - 1] = Tr::cvt(dp[mb][i - 1]);
         sb[E / 8][E % 8] = Tr::cvt(dsv);

@@ -102,6 +102,9 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   if (kBias)
     bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)h * a.sb_h +
            (int64_t)row_c * a.sb_m;
+  // 8-byte bias loads need unit column stride and 8-byte aligned rows
+  const bool bias_vec = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 3) == 0 &&
+                        (reinterpret_cast<uintptr_t>(a.bias) & 7) == 0;
 
   DropoutState ds{};
   if (kDropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
@@ -221,14 +224,26 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
         for (int i = 0; i < 16; ++i) s[mb][i] *= qk_scale;
     }
     if (kBias) {
+      if (bias_vec && (j + 1) * BN <= si.seqlen_k) {
+        // a lane's four consecutive keys of every 8-key group in one 8-byte load
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          int n = j * BN + mb * 32 + 8 * (i / 4) + 4 * hi + (i % 4);
-          n = n < si.seqlen_k ? n : si.seqlen_k - 1;
-          s[mb][i] += (float)bptr[(int64_t)n * a.sb_n] * kLog2e;   // fwd_kernel_inner.py:187
-        }
+          for (int g = 0; g < 4; ++g) {
+            const q4_t b4 = *reinterpret_cast<const q4_t*>(bptr + j * BN + mb * 32 + 8 * g + 4 * hi);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[mb][4 * g + r] += (float)b4[r] * kLog2e;   // fwd_kernel_inner.py:187
+          }
+      } else {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            int n = j * BN + mb * 32 + 8 * (i / 4) + 4 * hi + (i % 4);
+            n = n < si.seqlen_k ? n : si.seqlen_k - 1;
+            s[mb][i] += (float)bptr[(int64_t)n * a.sb_n] * kLog2e;   // fwd_kernel_inner.py:187
+          }
+      }
     }
     if (masked) {
 #pragma unroll
