@@ -61,9 +61,11 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
 // the transposing reads of the GEMMs that contract over the tile's rows, both free
 // of bank conflicts.  Q and dO (dK/dV item) and K (dQ item) are read both ways.
 template <int D, int BM>
-struct DkDvSmem {   // per stage: Q, dO (swizzled, one copy each); L, delta
+struct DkDvSmem {   // per stage: Q, dO (swizzled, one copy each); L, delta; bias tile (BM x 128 keys)
   static constexpr int TILE_BYTES = BM * D * 2;
-  static constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * BM * 4;
+  static constexpr int BIAS_STR = 128 * 2 + 16;       // bytes per bias row: rows 4 apart land 16 banks apart
+  static constexpr int BIAS_BYTES = BM * BIAS_STR;
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * BM * 4 + BIAS_BYTES;
   static constexpr int STAGES = 2;
   static constexpr int BYTES = STAGES * STAGE_BYTES;
 };
@@ -201,7 +203,20 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     lse_b = a.lse + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
     if (!kInlineDelta) delta_b = a.delta + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
   };
-  __amdgpu_buffer_rsrc_t q_rs, do_rs, o_rs;
+  __amdgpu_buffer_rsrc_t q_rs, do_rs, o_rs, b_rs;
+  // The bias tile (BM queries x the workgroup's 128 keys) is staged through LDS like Q
+  // and dO when its layout allows 16-byte loads; otherwise elements are loaded directly.
+  static_assert(BN == 128, "bias staging assumes 128 keys per workgroup");
+  constexpr int CHB = kBias ? (BM * 16) / NT : 0;        // 16-byte bias pieces per thread
+  const bool bias_lds = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 7) == 0 &&
+                        (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0;
+  op_t bch[CHB > 0 ? CHB : 1];
+  const int b_voff = (tid / 16) * (int)a.sb_m * 2 + (tid % 16) * 16;   // bytes inside a bias tile
+  const int b_soff = (NT / 16) * (int)a.sb_m * 2;
+  const int b_lds = (tid / 16) * SM::BIAS_STR + (tid % 16) * 16;
+  const T* bb = nullptr;
+  const T* bb_tile = nullptr;     // bias tile being fetched, its valid rows
+  int b_rows = 0;
   // (g, e) = (q-head inside the GQA group, Q tile inside the range) of the tile to fetch;
   // called for consecutive tiles only; `live` false: nothing is fetched
   auto fetch_begin = [&](bool live, int g, int e) {
@@ -210,6 +225,17 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     int rows = si.seqlen_q - m0 < BM ? si.seqlen_q - m0 : BM;
     rows = live ? rows : 0;
     const bool any = rows > 0;
+    if (kBias) {
+      if (live && e == 0)
+        bb = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
+             (int64_t)(hk * group + g) * a.sb_h + (int64_t)br.lo * BM * a.sb_m + (int64_t)n0 * a.sb_n;
+      bb_tile = bb;
+      b_rows = rows;
+      const int cols = si.seqlen_k - n0 < BN ? si.seqlen_k - n0 : BN;
+      b_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(bb), 0,
+                                               any && bias_lds ? ((rows - 1) * (int)a.sb_m + cols) * 2 : 0, 0x00020000);
+      if (live) bb += (int64_t)BM * a.sb_m;
+    }
     q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + D) * 2 : 0,
                                              0x00020000);
     do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
@@ -227,9 +253,24 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       if (kInlineDelta) ob += o_tile_step; else delta_b += BM;
     }
   };
-  constexpr int FETCH_PIECES = 2 * CH;
-  auto fetch_piece = [&](int i) {        // Q pieces first, then dO (and O)
-    if (i < CH) {
+  constexpr int FETCH_PIECES = 2 * CH + CHB;
+  auto fetch_piece = [&](int i) {        // Q pieces first, then dO (and O), then bias
+    if (i >= 2 * CH) {
+      const int k = i - 2 * CH;
+      if (bias_lds) {
+        bch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_voff, k * b_soff, 0));
+      } else {
+        // any other layout: the piece is gathered element by element
+        const int row = tid / 16 + k * (NT / 16), col = (tid % 16) * 8;
+        op_t x;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const bool ok = row < b_rows && n0 + col + e < si.seqlen_k;
+          x[e] = ok ? bb_tile[(int64_t)row * a.sb_m + (int64_t)(col + e) * a.sb_n] : Tr::cvt(0.f);
+        }
+        bch[k] = x;
+      }
+    } else if (i < CH) {
       qch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(q_rs, q_voff, i * q_soff, 0));
     } else {
       const int k = i - CH;
@@ -238,10 +279,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         och[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(o_rs, o_voff, k * o_soff, 0));
     }
   };
-  constexpr int STORE_PIECES = 2 * CH;
+  constexpr int STORE_PIECES = 2 * CH + CHB;
   auto store_piece = [&](int i, int stage) {   // same order as the fetches
     char* sp = stage_ptr(stage);
-    if (i < CH) *reinterpret_cast<op_t*>(sp + lds_off[i]) = qch[i];
+    if (i >= 2 * CH)
+      *reinterpret_cast<op_t*>(sp + 2 * SM::TILE_BYTES + 2 * BM * 4 + b_lds + (i - 2 * CH) * (NT / 16) * SM::BIAS_STR) =
+          bch[i - 2 * CH];
+    else if (i < CH) *reinterpret_cast<op_t*>(sp + lds_off[i]) = qch[i];
     else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = doch[i - CH];
   };
   auto store_stats = [&](int stage) {
@@ -278,21 +322,19 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const char* dOb = sp + SM::TILE_BYTES;
     const float* Ls = reinterpret_cast<const float*>(sp + 2 * SM::TILE_BYTES);
     const float* Ds = Ls + BM;
+    // this lane's key column of the staged bias tile
+    const T* Bs = reinterpret_cast<const T*>(sp + 2 * SM::TILE_BYTES + 2 * BM * 4) + wave * 32 + c;
 
     f32x16 s[MB], dp[MB];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     DropoutState dst{};
     if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
-    const T* bptr = nullptr;
-    if (kBias)
-      bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)hq * a.sb_h +
-             (int64_t)key_c * a.sb_n;
 
     // The vector ALU work is spread over the MFMAs of the GEMMs that do not depend on
     // it: p = exp2(...) of S runs behind the MFMAs of dP, ds = p (dP - delta) behind
     // those of dV.  Fences keep the hand-made order.
-    constexpr int kAhead = 2;
+    constexpr int kAhead = D >= 256 ? 1 : 2;
     op_t xa[kAhead + 1][MB];
     op_t pb[TS], sb[TS];
     // row statistics are read four rows at a time, one read ahead of their use
@@ -343,8 +385,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
       float x;
       if (kBias) {
-        const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
-        x = __builtin_fmaf(s[mb][i], qk_scale, (float)bptr[(int64_t)mm * a.sb_m] * kLog2e) - l4[(E / 4) & 1][r];
+        // rows of a full tile are all inside the sequence; offsets inside a tile fit 32 bits
+        const int ml = 32 * mb + 8 * g + r;
+        const float bv = (float)Bs[(ml + 4 * hi) * (SM::BIAS_STR / 2)];
+        x = __builtin_fmaf(s[mb][i], qk_scale, bv * kLog2e) - l4[(E / 4) & 1][r];
       } else {
         x = __builtin_fmaf(s[mb][i], qk_scale, -l4[(E / 4) & 1][r]);
       }
@@ -567,14 +611,28 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
             (int64_t)row_c * a.sdb_m;
   const int nkt = (si.seqlen_k + BN - 1) / BN;
 
-  // dB of K tiles that are never visited is zero
+  // dB of K tiles that are never visited is zero.  The wave sweeps its 32 rows; along a
+  // row the 64 lanes write 16 bytes each when the layout allows it.
   auto zero_db = [&](int j_from, int j_to) {
-    if (!(kBias && dbptr != nullptr && row_ok)) return;
-    for (int j = j_from; j < j_to; ++j)
-      for (int i = hi; i < BN; i += 2) {
-        const int n = j * BN + i;
-        if (n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(0.f);
+    if (!(kBias && a.db != nullptr)) return;
+    const int c0 = j_from * BN, c1 = j_to * BN < si.seqlen_k ? j_to * BN : si.seqlen_k;
+    if (c0 >= c1) return;
+    T* dbase = reinterpret_cast<T*>(a.db) + (int64_t)si.batch_index * a.sdb_z + (int64_t)h * a.sdb_h;
+    const bool vec = a.sdb_n == 1 && ((a.sdb_m | a.sdb_h | a.sdb_z) & 7) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.db) & 15) == 0;
+    const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int rr = 0; rr < 32; ++rr) {
+      const int m = q0 + wave * 32 + rr;
+      if (m >= si.seqlen_q) break;
+      T* rowp = dbase + (int64_t)m * a.sdb_m;
+      if (vec) {
+        const int v0 = (c0 + 7) & ~7, v1 = c1 & ~7;      // 16-byte aligned body (c0 is a multiple of BN)
+        for (int n = v0 + lane * 8; n < v1; n += 64 * 8) *reinterpret_cast<op_t*>(rowp + n) = zero8;
+        for (int n = (v1 > v0 ? v1 : c0) + lane; n < c1; n += 64) rowp[n] = Tr::cvt(0.f);
+      } else {
+        for (int n = c0 + lane; n < c1; n += 64) rowp[(int64_t)n * a.sdb_n] = Tr::cvt(0.f);
       }
+    }
   };
 
   if (br.lo > br.hi) {
@@ -699,7 +757,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     // The vector ALU work is spread over MFMAs that do not depend on it: p = exp2(...)
     // of S runs behind the MFMAs of dP, ds = p (dP - delta) of one 16-key step behind
     // the dQ MFMAs of the step before.  Fences keep the hand-made order.
-    constexpr int kAhead = 2;
+    constexpr int kAhead = D >= 256 ? 1 : 2;
     op_t xa[kAhead + 1][MB];
     op_t sb[TS];
     uint32_t keep[kDropout ? 4 * MB : 1];

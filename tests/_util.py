@@ -17,7 +17,7 @@ FUDGE = dict(out=3.0, dq=148.0, dk=48.0, dv=36.0, db=17.0)
 LSE_ATOL = 2e-3
 
 
-def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False):
+def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False, bias_layout='padded'):
     g = torch.Generator(device='cpu').manual_seed(seed)
 
     def rn(*shape, scale=1.0):
@@ -32,8 +32,11 @@ def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=Fa
         q = rn(B, Hq, Sq, D); k = rn(B, Hk, Sk, D); v = rn(B, Hk, Sk, D); do = rn(B, Hq, Sq, D)
     b = None
     if bias:
-        sk8 = (Sk + 7) // 8 * 8      # rows padded to 8 then sliced (_common_test.py:197-199)
-        b = rn(B, Hq, Sq, sk8, scale=0.5)[:, :, :, :Sk]
+        if bias_layout == 'padded':
+            sk8 = (Sk + 7) // 8 * 8      # rows padded to 8 then sliced (_common_test.py:197-199)
+            b = rn(B, Hq, Sq, sk8, scale=0.5)[:, :, :, :Sk]
+        else:                            # 'odd': odd row stride and a base that is only 2-byte aligned
+            b = rn(B, Hq, Sq, Sk + 3, scale=0.5)[:, :, :, 1:Sk + 1]
     return q, k, v, b, do
 
 

@@ -16,15 +16,16 @@ DEV = 'cuda'
 
 
 def _run_case(B, Hq, Hk, Sq, Sk, D, dtype, causal, dropout_p=0.0, bias=False, bshd=False,
-              bwd_backend=-1, sm_scale=None, seed=0):
+              bwd_backend=-1, sm_scale=None, seed=0, bias_layout='padded'):
     from aotriton_amd import flash
     from aotriton_amd.autograd import attention, AttentionExtraArgs
     from oracle import fa_ref
-    q, k, v, b, do = make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, DEV, seed=seed, bias=bias, bshd=bshd)
+    q, k, v, b, do = make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, DEV, seed=seed, bias=bias, bshd=bshd,
+                                 bias_layout=bias_layout)
     sm_scale = 1.0 / math.sqrt(D) if sm_scale is None else sm_scale
     ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=bwd_backend)
     qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
-    bg = b.clone().requires_grad_() if b is not None else None
+    bg = b.detach().requires_grad_() if b is not None else None      # keeps the strides of b
     o, _, L = attention(qg, kg, vg, bg, causal, sm_scale, dropout_p, ext)
     o.backward(do)
     torch.cuda.synchronize()
@@ -83,6 +84,12 @@ def test_dropout(D, causal, backend):
 @pytest.mark.parametrize('backend', [0, 1])
 def test_bias_and_db(D, causal, backend):
     _run_case(2, 3, 3, 150, 201, D, torch.float16, causal, bias=True, bwd_backend=backend)
+
+
+@pytest.mark.parametrize('backend', [0, 1])
+def test_bias_rows_without_vector_alignment(backend):
+    # bias whose rows are not 8- or 16-byte aligned: the kernels fall back to element access
+    _run_case(2, 2, 2, 150, 201, 128, torch.float16, (40, 0), bias=True, bwd_backend=backend, bias_layout='odd')
 
 
 def test_window_bias_dropout_small_config5():
