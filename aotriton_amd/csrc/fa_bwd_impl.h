@@ -337,6 +337,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     constexpr int kAhead = D >= 256 ? 1 : 2;
     op_t xa[kAhead + 1][MB];
     op_t pb[TS], sb[TS];
+    uint32_t kw[kDropout ? MB : 1][4];
     // row statistics are read four rows at a time, one read ahead of their use
     f32x4 l4[2], d4[2];
     auto stat_ptr = [&](const float* base, int q) { return base + 32 * (q / 4) + 8 * (q % 4) + 4 * hi; };
@@ -360,6 +361,18 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
         const int gidx = k * MB + mb;
         if (gidx == 0) fetch_begin(live, g_nxt, e_nxt);
+        if (kDropout) {
+          // One Philox call yields the keep bits of 4 consecutive keys, i.e. of the 4
+          // lanes of a quad, for one row: quad lane q runs the calls of the rows with
+          // m % 4 == q (8 per tile of 64 rows instead of 32) and the bits are exchanged
+          // with quad broadcasts when they are used.
+          constexpr int calls = 4 * MB, stride = G1 / calls > 0 ? G1 / calls : 1;
+          if (gidx % stride == 0 && gidx / stride < calls) {
+            const int cidx = gidx / stride;
+            kw[cidx / 4][cidx % 4] =
+                dropout_keep4(dst, m0 + 32 * (cidx / 4) + 8 * (cidx % 4) + 4 * hi + (lane & 3), key & ~3);
+          }
+        }
         if (gidx % every == every - 1) {
 #pragma unroll
           for (int q = 0; q < (FETCH_PIECES + G1 - 1) / G1; ++q) {
@@ -399,17 +412,25 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       }
       s[mb][i] = fast_exp2(x);
     };
+    // keep bit of element E: held by the quad lane that ran the Philox call of its row
+    auto keep_of = [&](int E) -> bool {
+      const int mb = E / 16, g = (E % 16) / 4, r = E % 4;
+      const int w = (int)kw[mb][g];
+      int w4;
+      switch (r) {       // quad_perm: [r, r, r, r]
+        case 0: w4 = __builtin_amdgcn_mov_dpp(w, 0x00, 0xf, 0xf, true); break;
+        case 1: w4 = __builtin_amdgcn_mov_dpp(w, 0x55, 0xf, 0xf, true); break;
+        case 2: w4 = __builtin_amdgcn_mov_dpp(w, 0xaa, 0xf, 0xf, true); break;
+        default: w4 = __builtin_amdgcn_mov_dpp(w, 0xff, 0xf, 0xf, true); break;
+      }
+      return ((uint32_t)w4 >> (lane & 3)) & 1u;
+    };
     bool keep_bit[kDropout ? 16 * MB : 1];
     auto p_pair = [&](int E) {   // E odd: operand form of (E-1, E); dropout applies to the operand only
       float p0 = s[E / 16][E % 16 - 1], p1 = s[E / 16][E % 16];
       if (kDropout) {
-        const int mb = E / 16;
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          const int i = E % 16 - 1 + q;
-          const int m = m0 + 32 * mb + 8 * (i / 4) + 4 * hi + (i % 4);
-          keep_bit[E - 1 + q] = dropout_keep1(dst, m, key);
-        }
+        keep_bit[E - 1] = keep_of(E - 1);
+        keep_bit[E] = keep_of(E);
         p0 = keep_bit[E - 1] ? p0 * dst.scale : 0.f;              // :200-201
         p1 = keep_bit[E] ? p1 * dst.scale : 0.f;
       }
