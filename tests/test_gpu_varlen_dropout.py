@@ -191,3 +191,66 @@ def test_headline_size_properties():
         colsum = vg.grad.float().sum(dim=2)
         dosum = do.float().sum(dim=2)
         assert (colsum - dosum).abs().max().item() < 0.5, (colsum - dosum).abs().max().item()
+
+
+@pytest.mark.parametrize('layout', ['padded', 'strided'])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_padded_and_strided_varlen(layout, causal, backend):
+    # varlen_type 2: rank-4 batch tensors padded to the longest sequence, LSE (n*Hq, max_sq);
+    # varlen_type 3: packed tokens with gaps, sequence starts from seq_strides, LSE (Hq, total)
+    # (modules/flash/kernel/fwd_kernel.py:243-286, tests/varlen_attn_torch_function.py:52-84).
+    from aotriton_amd import flash
+    from oracle import fa_ref
+    dtype, D, Hq, Hk = torch.bfloat16, 128, 4, 2
+    lens = np.array([70, 5, 192, 133])
+    pads = np.array([3, 11, 0, 60])
+    n, mx = len(lens), int(lens.max())
+    g = torch.Generator().manual_seed(11)
+    rn = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)
+    cu = torch.tensor([0] + np.cumsum(lens).tolist(), dtype=torch.int32, device=DEV)
+    if layout == 'padded':
+        q, k, v, do = rn(n, Hq, mx, D), rn(n, Hk, mx, D), rn(n, Hk, mx, D), rn(n, Hq, mx, D)
+        L = torch.zeros(n * Hq, mx, device=DEV, dtype=torch.float32)
+        ss = None
+        starts = [0] * n
+        sl = lambda t, i: t[i:i + 1, :, :lens[i]]
+    else:
+        T = int((lens + pads).sum())
+        q, k, v, do = rn(1, Hq, T, D), rn(1, Hk, T, D), rn(1, Hk, T, D), rn(1, Hq, T, D)
+        L = torch.zeros(Hq, T, device=DEV, dtype=torch.float32)
+        ss = torch.tensor([0] + np.cumsum(lens + pads).tolist(), dtype=torch.int32, device=DEV)
+        starts = ss.tolist()
+        sl = lambda t, i: t[:, :, starts[i]:starts[i] + lens[i]]
+    nan = float('nan')
+    o = torch.full_like(q, nan); dq = torch.full_like(q, nan); dk = torch.full_like(k, nan); dv = torch.full_like(v, nan)
+    delta = torch.zeros_like(L)
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+    sm = 1.0 / math.sqrt(D)
+    ok = flash.hipError_t.hipSuccess
+    assert flash.attn_fwd_varlen(q, k, v, cu, cu, mx, mx, ss, ss, None, sm, L, o, 0.0, null, null, 0, null, null,
+                                 None, causal, atomic, layout) == ok
+    ext = flash.attn_options(); ext.force_backend_index = backend
+    assert flash.attn_bwd_varlen(q, k, v, cu, cu, mx, mx, ss, ss, None, sm, o, do, dq, dk, dv, None, None, L, delta,
+                                 0.0, null, null, 0, causal, layout, extargs=ext) == ok
+    torch.cuda.synchronize()
+    ct, wl, wr = flash.translate_causal(causal)
+    f = lambda t: t.float()
+    for i in range(n):
+        qi, ki, vi, doi = sl(q, i), sl(k, i), sl(v, i), sl(do, i)
+        ro, rl, _ = fa_ref.attn_fwd_ref(f(qi), f(ki), f(vi), None, sm, ct, wl, wr, 0.0, None)
+        lo, ll, _ = fa_ref.attn_fwd_ref(qi, ki, vi, None, sm, ct, wl, wr, 0.0, None)
+        check(f'out[{i}]', sl(o, i), ro, lo, FUDGE['out'])
+        Li = L.view(n, Hq, mx)[i:i + 1, :, :lens[i]] if layout == 'padded' else L[None, :, starts[i]:starts[i] + lens[i]]
+        assert (Li - rl).abs().max().item() <= LSE_ATOL
+        rg = fa_ref.attn_bwd_ref(f(qi), f(ki), f(vi), None, sm, ro, f(doi), rl, ct, wl, wr, 0.0, None)
+        lg = fa_ref.attn_bwd_ref(qi, ki, vi, None, sm, lo, doi, ll.to(dtype).float().to(dtype), ct, wl, wr, 0.0, None)
+        check(f'dq[{i}]', sl(dq, i), rg[0], lg[0], FUDGE['dq'])
+        check(f'dk[{i}]', sl(dk, i), rg[1], lg[1], FUDGE['dk'])
+        check(f'dv[{i}]', sl(dv, i), rg[2], lg[2], FUDGE['dv'])
+    # rows outside the sequences are never written
+    if layout == 'padded':
+        assert torch.isnan(o[1, :, lens[1]:]).all() and torch.isnan(dk[1, :, lens[1]:]).all()
+    else:
+        assert torch.isnan(o[:, :, lens[0]:starts[1]]).all() and torch.isnan(dv[:, :, lens[0]:starts[1]]).all()
