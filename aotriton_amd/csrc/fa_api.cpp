@@ -90,7 +90,7 @@ fa::Strides3 strides3(const fa_tensor4& t) {
 }
 
 struct Shape {
-  int batch, hq, hk, d, max_sq, max_sk, num_seqlens;  // num_seqlens signed as in attn_fwd.cc:99
+  int batch, hq, hk, d, d_act, max_sq, max_sk, num_seqlens;  // d: compiled head dim, d_act: the tensors'; num_seqlens signed as in attn_fwd.cc:99
   bool windowed, bias, dropout;
 };
 
@@ -117,9 +117,11 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   if (s.hk <= 0 || s.hq <= 0 || s.hq % s.hk != 0 || (int)V.sizes[1] != s.hk) return FA_ERROR_INVALID_VALUE;
   if (K.sizes[0] != Q.sizes[0] || V.sizes[0] != Q.sizes[0]) return FA_ERROR_INVALID_VALUE;
   if (K.sizes[2] != V.sizes[2]) return FA_ERROR_INVALID_VALUE;
-  // compiled head dims; padded / mixed head dims are not built (attn_fwd.cc:76-82)
-  if (dqk != dv || !(dqk == 64 || dqk == 128 || dqk == 256)) return FA_ERROR_NOT_SUPPORTED;
-  s.d = dqk;
+  // Head dims are rounded up to a compiled one and the excess columns are masked in
+  // the kernels (PADDED_HEAD, attn_fwd.cc:76-82,109); 16-byte granularity, Dqk = Dv.
+  if (dqk != dv || dqk <= 0 || dqk > 256 || dqk % 8 != 0) return FA_ERROR_NOT_SUPPORTED;
+  s.d_act = dqk;
+  s.d = dqk <= 64 ? 64 : (dqk <= 128 ? 128 : 256);
   s.max_sq = (int)Q.sizes[2];
   s.max_sk = (int)K.sizes[2];
   s.num_seqlens = 0;
@@ -413,7 +415,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
     a.sb_z = (int64_t)p->B.strides[0]; a.sb_h = (int64_t)p->B.strides[1];
     a.sb_m = (int64_t)p->B.strides[2]; a.sb_n = (int64_t)p->B.strides[3];
   }
-  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk;
+  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_act;
   a.sm_scale = p->Sm_scale;
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
@@ -471,7 +473,7 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
     a.sdb_z = (int64_t)p->DB.strides[0]; a.sdb_h = (int64_t)p->DB.strides[1];
     a.sdb_m = (int64_t)p->DB.strides[2]; a.sdb_n = (int64_t)p->DB.strides[3];
   }
-  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk;
+  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_act;
   a.sm_scale = p->Sm_scale;
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};

@@ -252,6 +252,10 @@ __device__ __forceinline__ SeqInfo get_seq(const SeqArgs& s, int z) {
   return r;
 }
 
+// Byte offset that no buffer descriptor of these kernels covers: a lane whose 16-byte
+// chunk lies in the padding of a head dim that was rounded up reads zeros with it.
+constexpr int kVoffOutOfRange = 0x7fff0000;
+
 // (sequence, head) of the linear work index zh.  The heads of one GQA group are
 // adjacent, then come the sequences, then the kv-heads: the contiguous range of zh
 // that an XCD owns then holds whole kv-heads across ALL sequences, so XCDs get equal

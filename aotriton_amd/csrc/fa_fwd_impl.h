@@ -52,6 +52,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
+  const int d_act = a.head_dim;          // <= D, multiple of 8
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * BM;
@@ -81,7 +82,8 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = zero4;
+        for (int g = 0; g < 4; ++g)
+          if (32 * db + 8 * g + 4 * hi < d_act) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = zero4;
       if (lse_ptr && hi == 0) lse_ptr[row] = __builtin_inff();
     }
     return;
@@ -92,7 +94,11 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
                   (int64_t)h * a.sq.h + (int64_t)(si.q_start + row_c) * a.sq.s;
   op_t qreg[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const op_t*>(qptr + 16 * ks + 8 * hi);
+  for (int ks = 0; ks < KS; ++ks) {
+    // columns past the tensors' head dim are zero (head dims are rounded up to D)
+    const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    qreg[ks] = 16 * ks + 8 * hi < d_act ? *reinterpret_cast<const op_t*>(qptr + 16 * ks + 8 * hi) : zero8;
+  }
 
   const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
                    (int64_t)hk * a.sk.h + (int64_t)si.k_start * a.sk.s;
@@ -120,8 +126,9 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   static_assert(NT % LPR == 0, "threads must cover whole rows");
   op_t kreg[CH], vreg[CH];
   const int r0 = tid / LPR, cc0 = tid % LPR;
-  const int kvoff = r0 * (int)a.sk.s * 2 + cc0 * 16;      // bytes inside a tile
-  const int vvoff = r0 * (int)a.sv.s * 2 + cc0 * 16;
+  const bool col_ok = cc0 * 8 < d_act;
+  const int kvoff = col_ok ? r0 * (int)a.sk.s * 2 + cc0 * 16 : kVoffOutOfRange;      // bytes inside a tile
+  const int vvoff = col_ok ? r0 * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
   const int ksoff = RPI * (int)a.sk.s * 2, vsoff = RPI * (int)a.sv.s * 2;
   const int ldsk0 = r0 * KSTR + cc0 * 8, ldsv0 = r0 * VSTR + cc0 * 8;   // elements
 
@@ -134,9 +141,9 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   int rows_left = si.seqlen_k - br.lo * BN;      // > 0
   auto load_next_tile = [&]() {
     const int rows = rows_left < BN ? rows_left : BN;
-    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, (rows - 1) * k_row_bytes + D * 2,
+    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, (rows - 1) * k_row_bytes + d_act * 2,
                                                        0x00020000);
-    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, (rows - 1) * v_row_bytes + D * 2,
+    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, (rows - 1) * v_row_bytes + d_act * 2,
                                                        0x00020000);
 #pragma unroll
     for (int i = 0; i < CH; ++i)
@@ -410,7 +417,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
         q4_t t4;
 #pragma unroll
         for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(o[db][4 * g + r] * inv);
-        *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
+        if (32 * db + 8 * g + 4 * hi < d_act) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
       }
     if (lse_ptr && hi == 0)
       lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612

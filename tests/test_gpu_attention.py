@@ -97,6 +97,19 @@ def test_window_bias_dropout_small_config5():
     _run_case(1, 2, 2, 384, 384, 256, torch.float16, (100, 0), dropout_p=0.1, bias=True)
 
 
+@pytest.mark.parametrize('D', [16, 40, 80, 96, 160, 192, 224])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_head_dims_rounded_up(D, causal, backend):
+    # head dims between the compiled ones run on the next larger kernel with the excess
+    # columns masked (the reference's PADDED_HEAD, modules/flash/csrc/attn_fwd.cc:76-82,109)
+    _run_case(2, 4, 2, 203, 171, D, torch.bfloat16, causal, bwd_backend=backend, bshd=(D % 32 == 0))
+
+
+def test_head_dim_rounded_up_with_bias_dropout_varlen_strides():
+    _run_case(1, 2, 2, 130, 130, 72, torch.float16, (30, 0), dropout_p=0.3, bias=True)
+
+
 @pytest.mark.parametrize('causal', [1, 2])
 def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
     # rows with no visible key: O = 0, LSE = +inf, gradients finite

@@ -102,7 +102,12 @@ def test_validate_fwd_error_contract():
     assert validate_fwd(p, attn_fwd_params.kVersion) == E.hipSuccess
     assert validate_fwd(p, 2) == E.hipErrorInvalidSymbol                       # version gate
     p2, k2 = _fwd_params(D=96)
-    assert validate_fwd(p2, 3) == E.hipErrorNotSupported                       # head dim not built
+    assert validate_fwd(p2, 3) == E.hipSuccess                                 # rounded up to 128, columns masked
+    err, cfg = query_fwd_config(p2)
+    assert err == E.hipSuccess and cfg.head_dim == 128
+    for bad in (512, 100):                                                     # > 256, or rows not a multiple of 16 bytes
+        pb, kb = _fwd_params(D=bad)
+        assert validate_fwd(pb, 3) == E.hipErrorNotSupported
     p3, k3 = _fwd_params(dtype=torch.float32)
     assert validate_fwd(p3, 3) == E.hipErrorNotSupported                       # fp32 kernels not built
     p4, k4 = _fwd_params(Hq=5, Hk=2)
