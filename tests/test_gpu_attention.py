@@ -146,3 +146,49 @@ def test_row_maximum_grows_along_keys(dtype, causal):
     check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
     check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
     check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
+
+
+@pytest.mark.parametrize('mode', ['plain', 'causal', 'float_mask', 'bool_mask', 'gqa_bshd'])
+def test_sdpa_entry_point_matches_torch_math(mode):
+    # the F.scaled_dot_product_attention-shaped entry point against PyTorch's math SDPA in fp32
+    import torch.nn.functional as F
+    from torch.nn.attention import sdpa_kernel, SDPBackend
+    from aotriton_amd.sdpa import scaled_dot_product_attention as sdpa
+    B, H, L, S, E = 2, 4, 150, 201, 96
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)
+    hk = 2 if mode == 'gqa_bshd' else H
+    if mode == 'gqa_bshd':
+        q, k, v = rn(B, L, H, E).transpose(1, 2), rn(B, S, hk, E).transpose(1, 2), rn(B, S, hk, E).transpose(1, 2)
+    else:
+        q, k, v = rn(B, H, L, E), rn(B, hk, S, E), rn(B, hk, S, E)
+    kw = {}
+    if mode == 'causal':
+        kw['is_causal'] = True
+    elif mode == 'float_mask':
+        kw['attn_mask'] = rn(1, 1, L, S) * 0.5            # broadcast over batch and heads
+    elif mode == 'bool_mask':
+        keep = torch.rand(B, 1, L, S, generator=g) > 0.3
+        keep[..., 0] = True                                # no fully hidden row
+        kw['attn_mask'] = keep.to(DEV)
+    elif mode == 'gqa_bshd':
+        kw['enable_gqa'] = True
+    do = rn(*q.shape) if mode != 'gqa_bshd' else rn(B, L, H, E).transpose(1, 2)
+    outs, grads = [], []
+    for fn, cast in ((sdpa, lambda t: t), (F.scaled_dot_product_attention, lambda t: t.float()),
+                     (F.scaled_dot_product_attention, lambda t: t)):
+        qq, kk, vv = [cast(t).detach().clone().requires_grad_() for t in (q, k, v)]
+        kw2 = dict(kw)
+        if 'attn_mask' in kw2 and kw2['attn_mask'].dtype != torch.bool:
+            kw2['attn_mask'] = cast(kw2['attn_mask'])
+        if fn is sdpa:
+            o = fn(qq, kk, vv, **kw2)
+        else:
+            with sdpa_kernel(SDPBackend.MATH):
+                o = fn(qq, kk, vv, **kw2)
+        o.backward(cast(do))
+        outs.append(o); grads.append((qq.grad, kk.grad, vv.grad))
+    check('out', outs[0], outs[1], outs[2], FUDGE['out'])
+    for name, i in (('dq', 0), ('dk', 1), ('dv', 2)):
+        check(name, grads[0][i], grads[1][i], grads[2][i], FUDGE[name])
