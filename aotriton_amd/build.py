@@ -5,6 +5,7 @@ Usage: python -m aotriton_amd.build [-j N] [--force]
 import argparse
 import concurrent.futures
 import os
+import re
 import subprocess
 import sys
 
@@ -24,8 +25,28 @@ COMMON = [
 ]
 
 
+# Per-file additions.  The dQ kernels post-process MFMA results with the vector ALU; letting
+# the register allocator keep those results in VGPRs saves the AGPR read per element.
+EXTRA = {
+    'fa_bwd_dq_d64.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
+    'fa_bwd_dq_d128.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
+}
+
+# The per-head-dim kernel files are compiled a second time with FA_PADDED=1: the copies that
+# serve head dims rounded up to the compiled one.
+PADDED_RE = re.compile(r'fa_(fwd|bwd_dkdv|bwd_dq|bwd_fused)_d\d+\.hip$')
+
+
 def sources():
-    return sorted(f for f in os.listdir(CSRC) if f.endswith('.hip') or f.endswith('.cpp'))
+    """(source file, extra defines, object name) per compilation."""
+    out = []
+    for f in sorted(os.listdir(CSRC)):
+        if not (f.endswith('.hip') or f.endswith('.cpp')):
+            continue
+        out.append((f, [], f + '.o'))
+        if PADDED_RE.match(f):
+            out.append((f, ['-DFA_PADDED=1'], f + '.padded.o'))
+    return out
 
 
 def headers():
@@ -34,13 +55,14 @@ def headers():
     return hs
 
 
-def _compile(src, force):
-    obj = os.path.join(OBJ, src + '.o')
+def _compile(unit, force):
+    src, defines, objname = unit
+    obj = os.path.join(OBJ, objname)
     path = os.path.join(CSRC, src)
     newest = max(os.path.getmtime(p) for p in [path] + headers())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj, '', 0
-    cmd = [HIPCC] + COMMON + ['-x', 'hip', '-c', path, '-o', obj]
+    cmd = [HIPCC] + COMMON + EXTRA.get(src, []) + defines + ['-x', 'hip', '-c', path, '-o', obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature name; that note is noise
     err = '\n'.join(l for l in r.stderr.splitlines() if 'packed-fp32-ops' not in l)

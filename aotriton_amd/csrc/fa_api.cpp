@@ -248,10 +248,11 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
+  const bool padded = a.head_dim != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
-    case 64: return fa::run_fwd_d64(dtype, a, s.windowed, s.bias, s.dropout, stream);
-    case 128: return fa::run_fwd_d128(dtype, a, s.windowed, s.bias, s.dropout, stream);
-    case 256: return fa::run_fwd_d256(dtype, a, s.windowed, s.bias, s.dropout, stream);
+    case 64: return (padded ? fa::run_fwd_d64_padded : fa::run_fwd_d64)(dtype, a, s.windowed, s.bias, s.dropout, stream);
+    case 128: return (padded ? fa::run_fwd_d128_padded : fa::run_fwd_d128)(dtype, a, s.windowed, s.bias, s.dropout, stream);
+    case 256: return (padded ? fa::run_fwd_d256_padded : fa::run_fwd_d256)(dtype, a, s.windowed, s.bias, s.dropout, stream);
   }
   return hipErrorNotSupported;
 }

@@ -3,15 +3,21 @@
 
 namespace fa {
 
+// Tensors whose head dim is one of the compiled ones take the kernels with a constant head
+// dim; smaller head dims take the copies that mask the excess columns.
 #define FA_DECL(name)                                                                                   \
   hipError_t name##_d64(int, const BwdArgs&, bool, bool, bool, hipStream_t);                            \
   hipError_t name##_d128(int, const BwdArgs&, bool, bool, bool, hipStream_t);                           \
   hipError_t name##_d256(int, const BwdArgs&, bool, bool, bool, hipStream_t);                           \
+  hipError_t name##_d64_padded(int, const BwdArgs&, bool, bool, bool, hipStream_t);                     \
+  hipError_t name##_d128_padded(int, const BwdArgs&, bool, bool, bool, hipStream_t);                    \
+  hipError_t name##_d256_padded(int, const BwdArgs&, bool, bool, bool, hipStream_t);                    \
   hipError_t name(int dtype, int head_dim, const BwdArgs& a, bool w, bool b, bool p, hipStream_t s) {   \
+    const bool padded = a.head_dim != head_dim;                                                         \
     switch (head_dim) {                                                                                 \
-      case 64: return name##_d64(dtype, a, w, b, p, s);                                                 \
-      case 128: return name##_d128(dtype, a, w, b, p, s);                                               \
-      case 256: return name##_d256(dtype, a, w, b, p, s);                                               \
+      case 64: return padded ? name##_d64_padded(dtype, a, w, b, p, s) : name##_d64(dtype, a, w, b, p, s);    \
+      case 128: return padded ? name##_d128_padded(dtype, a, w, b, p, s) : name##_d128(dtype, a, w, b, p, s); \
+      case 256: return padded ? name##_d256_padded(dtype, a, w, b, p, s) : name##_d256(dtype, a, w, b, p, s); \
     }                                                                                                   \
     return hipErrorNotSupported;                                                                        \
   }

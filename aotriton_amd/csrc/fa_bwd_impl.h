@@ -86,7 +86,7 @@ template <> struct BwdTile<256> { static constexpr int NW = 4, DKDV_BM = 32, DQ_
 // ---------------------------------------------------------------------------
 // dK / dV work item
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta>
+template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta, bool kPad>
 __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const int nt, const int z,
                                           char* smem_raw) {
   using Tr = Traits<T>;
@@ -103,7 +103,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int d_act = a.head_dim;          // <= D, multiple of 8
+  const int d_act = kPad ? a.head_dim : D;   // <= D, multiple of 8; a constant unless the head dim is rounded up
 
   const SeqInfo si = get_seq(a.seq, z);
   const int n0 = nt * BN;
@@ -601,7 +601,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 // ---------------------------------------------------------------------------
 // dQ (+dB) work item
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta>
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta, bool kPad>
 __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int mt, const int z,
                                         char* smem_raw) {
   using Tr = Traits<T>;
@@ -617,7 +617,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int d_act = a.head_dim;          // <= D, multiple of 8
+  const int d_act = kPad ? a.head_dim : D;   // <= D, multiple of 8; a constant unless the head dim is rounded up
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * BM;
@@ -979,7 +979,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 // ---------------------------------------------------------------------------
 // Kernels
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout>
+template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dkdv_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -994,10 +994,10 @@ void bwd_dkdv_kernel(const BwdArgs a) {
   if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
   int z, hk;
   split_zh(zh, a.num_zh / a.hk, 1, z, hk);
-  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false>(a, hk, gr / a.zh_group, z, smem_raw);
+  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad>(a, hk, gr / a.zh_group, z, smem_raw);
 }
 
-template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dq_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -1011,7 +1011,7 @@ void bwd_dq_kernel(const BwdArgs a) {
   const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
   int z, h;
   split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
-  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false>(a, h, mt, z, smem_raw);
+  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false, kPad>(a, h, mt, z, smem_raw);
 }
 
 // Per (batch, kv-head): num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
@@ -1019,7 +1019,7 @@ void bwd_dq_kernel(const BwdArgs a) {
 // the same 1-D grid as the split kernels: each XCD owns a contiguous range of (batch,
 // kv-head) pairs and walks them in pairs, so the tensors of the heads in flight stay in
 // that XCD's L2.
-template <typename T, int D, int NW, int BM, int BN, bool kWindowed, bool kBias, bool kDropout>
+template <typename T, int D, int NW, int BM, int BN, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_fused_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -1035,12 +1035,12 @@ void bwd_fused_kernel(const BwdArgs a) {
   split_zh(zh, a.num_zh / a.hk, 1, z, hk);
   const int item = gr / a.zh_group;
   if (item < a.num_n_tiles) {
-    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true>(a, hk, item, z, smem_raw);
+    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true, kPad>(a, hk, item, z, smem_raw);
   } else {
     const int t = item - a.num_n_tiles;
     const int h = hk * group + t / a.num_m_tiles;
     const int mt = a.num_m_tiles - 1 - t % a.num_m_tiles;
-    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true>(a, h, mt, z, smem_raw);
+    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true, kPad>(a, h, mt, z, smem_raw);
   }
 }
 
@@ -1082,7 +1082,7 @@ hipError_t launch_bwd_preprocess(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <typename T, int D>
+template <typename T, int D, bool kPad>
 hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
   constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = NW * 32;
   BwdArgs a = a0;
@@ -1091,12 +1091,12 @@ hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dro
   a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
   a.zh_group = 2;
   dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles));
-#define FA_CALL(W, B, P) launch_with_lds(bwd_dkdv_kernel<T, D, NW, BM, W, B, P>, grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
+#define FA_CALL(W, B, P) launch_with_lds(bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>, grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
 
-template <typename T, int D>
+template <typename T, int D, bool kPad>
 hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
   constexpr int NW = BwdTile<D>::NW, BN = BwdTile<D>::DQ_BN, BM = NW * 32;
   BwdArgs a = a0;
@@ -1105,12 +1105,12 @@ hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropo
   a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
   a.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
   dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_m_tiles));
-#define FA_CALL(W, B, P) launch_with_lds(bwd_dq_kernel<T, D, NW, BN, W, B, P>, grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
+#define FA_CALL(W, B, P) launch_with_lds(bwd_dq_kernel<T, D, NW, BN, W, B, P, kPad>, grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
 
-template <typename T, int D>
+template <typename T, int D, bool kPad>
 hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
   constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = BwdTile<D>::DQ_BN;
   constexpr int smem = DkDvSmem<D, BM>::BYTES > DqSmem<D, BN>::BYTES ? DkDvSmem<D, BM>::BYTES : DqSmem<D, BN>::BYTES;
@@ -1122,7 +1122,7 @@ hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dr
   a.zh_group = 2;
   const int items = a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk);
   dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * items));
-#define FA_CALL(W, B, P) launch_with_lds(bwd_fused_kernel<T, D, NW, BM, BN, W, B, P>, grid, NW * 64, smem, stream, a)
+#define FA_CALL(W, B, P) launch_with_lds(bwd_fused_kernel<T, D, NW, BM, BN, W, B, P, kPad>, grid, NW * 64, smem, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }

@@ -2,9 +2,20 @@
 #include "fa_fwd_impl.h"
 #include "fa_kernels.h"
 
+// Compiled twice: as is for tensors whose head dim is 256, and with FA_PADDED=1 for smaller
+// head dims (a multiple of 8), where the kernels mask the excess columns.
+#ifndef FA_PADDED
+#define FA_PADDED 0
+#endif
+#if FA_PADDED
+#define FA_RUN run_fwd_d256_padded
+#else
+#define FA_RUN run_fwd_d256
+#endif
+
 namespace fa {
-hipError_t run_fwd_d256(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
-  if (dtype == kDtypeBF16) return launch_fwd<bf16_t, 256>(a, windowed, bias, dropout, s);
-  return launch_fwd<f16_t, 256>(a, windowed, bias, dropout, s);
+hipError_t FA_RUN(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
+  if (dtype == kDtypeBF16) return launch_fwd<bf16_t, 256, FA_PADDED != 0>(a, windowed, bias, dropout, s);
+  return launch_fwd<f16_t, 256, FA_PADDED != 0>(a, windowed, bias, dropout, s);
 }
 }  // namespace fa

@@ -31,7 +31,7 @@ struct FwdSmem {
 };
 
 // One Q tile (BM rows of head h of sequence z) against all its visible K/V tiles.
-template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const int h, const int mt, char* smem_raw) {
   using Tr = Traits<T>;
   using op_t = typename Tr::op_t;
@@ -52,7 +52,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int d_act = a.head_dim;          // <= D, multiple of 8
+  const int d_act = kPad ? a.head_dim : D;   // <= D, multiple of 8; a constant unless the head dim is rounded up
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * BM;
@@ -431,7 +431,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 // interleaved, and the workgroups of the XCD take them in serpentine order (worker p
 // takes p, 2P-1-p, 2P+p, ...), which pairs heavy with light tiles.  A workgroup
 // goes from one tile to the next without a relaunch.
-template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout>
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1, D <= 128 ? 2 : 1)))
 void fwd_kernel(const FwdArgs a) {
@@ -460,7 +460,7 @@ void fwd_kernel(const FwdArgs a) {
     const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
     int z, h;
     split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
-    fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout>(a, z, h, mt, smem_raw);
+    fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>(a, z, h, mt, smem_raw);
   }
 }
 
@@ -470,10 +470,10 @@ template <> struct FwdTile<64>  { static constexpr int NW = 8, BN = 64; };
 template <> struct FwdTile<128> { static constexpr int NW = 8, BN = 64; };
 template <> struct FwdTile<256> { static constexpr int NW = 4, BN = 32; };
 
-template <typename T, int D, bool kWindowed, bool kBias, bool kDropout>
+template <typename T, int D, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
   constexpr int NW = FwdTile<D>::NW, BN = FwdTile<D>::BN;
-  auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout>;
+  auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>;
   constexpr int smem = FwdSmem<D, BN>::BYTES;
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -484,7 +484,8 @@ hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <typename T, int D>
+// kPad: the tensors' head dim (FwdArgs::head_dim) is smaller than D and the excess columns are masked.
+template <typename T, int D, bool kPad>
 hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t stream) {
   constexpr int BM = FwdTile<D>::NW * 32;
   const int nseq = a.seq.num_seqlens != 0 ? (a.seq.num_seqlens < 0 ? -a.seq.num_seqlens : a.seq.num_seqlens)
@@ -502,14 +503,14 @@ hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, 
   dim3 grid((unsigned)(kNumXcd * workers));
   const int key = (windowed ? 4 : 0) | (bias ? 2 : 0) | (dropout ? 1 : 0);
   switch (key) {
-    case 0: return launch_fwd_variant<T, D, false, false, false>(b, grid, stream);
-    case 1: return launch_fwd_variant<T, D, false, false, true>(b, grid, stream);
-    case 2: return launch_fwd_variant<T, D, false, true, false>(b, grid, stream);
-    case 3: return launch_fwd_variant<T, D, false, true, true>(b, grid, stream);
-    case 4: return launch_fwd_variant<T, D, true, false, false>(b, grid, stream);
-    case 5: return launch_fwd_variant<T, D, true, false, true>(b, grid, stream);
-    case 6: return launch_fwd_variant<T, D, true, true, false>(b, grid, stream);
-    default: return launch_fwd_variant<T, D, true, true, true>(b, grid, stream);
+    case 0: return launch_fwd_variant<T, D, false, false, false, kPad>(b, grid, stream);
+    case 1: return launch_fwd_variant<T, D, false, false, true, kPad>(b, grid, stream);
+    case 2: return launch_fwd_variant<T, D, false, true, false, kPad>(b, grid, stream);
+    case 3: return launch_fwd_variant<T, D, false, true, true, kPad>(b, grid, stream);
+    case 4: return launch_fwd_variant<T, D, true, false, false, kPad>(b, grid, stream);
+    case 5: return launch_fwd_variant<T, D, true, false, true, kPad>(b, grid, stream);
+    case 6: return launch_fwd_variant<T, D, true, true, false, kPad>(b, grid, stream);
+    default: return launch_fwd_variant<T, D, true, true, true, kPad>(b, grid, stream);
   }
 }
 

@@ -13,6 +13,10 @@ struct TileShape { int block_m, block_n, num_waves, lds_bytes; };
 hipError_t run_fwd_d64(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_fwd_d128(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_fwd_d256(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+// the same kernels with the columns past FwdArgs::head_dim masked (head dims rounded up)
+hipError_t run_fwd_d64_padded(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_fwd_d128_padded(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_fwd_d256_padded(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 TileShape fwd_tile_shape(int head_dim);
 
 hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s);
