@@ -90,7 +90,7 @@ fa::Strides3 strides3(const fa_tensor4& t) {
 }
 
 struct Shape {
-  int batch, hq, hk, d, d_act, max_sq, max_sk, num_seqlens;  // d: compiled head dim, d_act: the tensors'; num_seqlens signed as in attn_fwd.cc:99
+  int batch, hq, hk, d, d_qk, d_v, max_sq, max_sk, num_seqlens;  // d: compiled head dim; d_qk, d_v: the tensors'; num_seqlens signed as in attn_fwd.cc:99
   bool windowed, bias, dropout;
 };
 
@@ -118,10 +118,13 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   if (K.sizes[0] != Q.sizes[0] || V.sizes[0] != Q.sizes[0]) return FA_ERROR_INVALID_VALUE;
   if (K.sizes[2] != V.sizes[2]) return FA_ERROR_INVALID_VALUE;
   // Head dims are rounded up to a compiled one and the excess columns are masked in
-  // the kernels (PADDED_HEAD, attn_fwd.cc:76-82,109); 16-byte granularity, Dqk = Dv.
-  if (dqk != dv || dqk <= 0 || dqk > 256 || dqk % 8 != 0) return FA_ERROR_NOT_SUPPORTED;
-  s.d_act = dqk;
-  s.d = dqk <= 64 ? 64 : (dqk <= 128 ? 128 : 256);
+  // the kernels (PADDED_HEAD, attn_fwd.cc:76-82,109); 16-byte granularity.  Dqk and Dv
+  // may differ: both run on the compiled head dim that holds the larger one.
+  if (dqk <= 0 || dqk > 256 || dqk % 8 != 0 || dv <= 0 || dv > 256 || dv % 8 != 0) return FA_ERROR_NOT_SUPPORTED;
+  s.d_qk = dqk;
+  s.d_v = dv;
+  const int dmax = dqk > dv ? dqk : dv;
+  s.d = dmax <= 64 ? 64 : (dmax <= 128 ? 128 : 256);
   s.max_sq = (int)Q.sizes[2];
   s.max_sk = (int)K.sizes[2];
   s.num_seqlens = 0;
@@ -224,7 +227,8 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   if ((e = check_act(p->DK, dt)) != FA_SUCCESS) return e;
   if ((e = check_act(p->DV, dt)) != FA_SUCCESS) return e;
   for (int i = 0; i < 4; ++i) {
-    if (p->Out.sizes[i] != p->Q.sizes[i] || p->DO.sizes[i] != p->Q.sizes[i] ||
+    const auto o_i = i == 3 ? p->V.sizes[3] : p->Q.sizes[i];
+    if (p->Out.sizes[i] != o_i || p->DO.sizes[i] != o_i ||
         p->DQ.sizes[i] != p->Q.sizes[i] || p->DK.sizes[i] != p->K.sizes[i] ||
         p->DV.sizes[i] != p->V.sizes[i])
       return FA_ERROR_INVALID_VALUE;
@@ -248,7 +252,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
-  const bool padded = a.head_dim != d;   // head dim rounded up: the copies that mask the excess columns
+  const bool padded = a.head_dim != d || a.head_dim_v != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
     case 64: return (padded ? fa::run_fwd_d64_padded : fa::run_fwd_d64)(dtype, a, s.windowed, s.bias, s.dropout, stream);
     case 128: return (padded ? fa::run_fwd_d128_padded : fa::run_fwd_d128)(dtype, a, s.windowed, s.bias, s.dropout, stream);
@@ -416,7 +420,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
     a.sb_z = (int64_t)p->B.strides[0]; a.sb_h = (int64_t)p->B.strides[1];
     a.sb_m = (int64_t)p->B.strides[2]; a.sb_n = (int64_t)p->B.strides[3];
   }
-  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_act;
+  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_qk; a.head_dim_v = s.d_v;
   a.sm_scale = p->Sm_scale;
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
@@ -474,7 +478,7 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
     a.sdb_z = (int64_t)p->DB.strides[0]; a.sdb_h = (int64_t)p->DB.strides[1];
     a.sdb_m = (int64_t)p->DB.strides[2]; a.sdb_n = (int64_t)p->DB.strides[3];
   }
-  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_act;
+  a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_qk; a.head_dim_v = s.d_v;
   a.sm_scale = p->Sm_scale;
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};

@@ -40,7 +40,8 @@ struct FwdArgs {
   Strides3 sq, sk, sv, so;
   int64_t sb_z, sb_h, sb_m, sb_n;
   int32_t batch, hq, hk;
-  int32_t head_dim;      // columns of the tensors (<= the compiled head dim, multiple of 8)
+  int32_t head_dim;      // columns of Q and K (<= the compiled head dim, multiple of 8)
+  int32_t head_dim_v;    // columns of V, Out and dOut (same bounds)
   float sm_scale;
   SeqArgs seq;
   MaskArgs mask;
@@ -64,7 +65,8 @@ struct BwdArgs {
   int64_t sb_z, sb_h, sb_m, sb_n;
   int64_t sdb_z, sdb_h, sdb_m, sdb_n;
   int32_t batch, hq, hk;
-  int32_t head_dim;      // columns of the tensors (<= the compiled head dim, multiple of 8)
+  int32_t head_dim;      // columns of Q and K (<= the compiled head dim, multiple of 8)
+  int32_t head_dim_v;    // columns of V, Out and dOut (same bounds)
   float sm_scale;
   SeqArgs seq;
   MaskArgs mask;

@@ -13,7 +13,7 @@ namespace fa {
   hipError_t name##_d128_padded(int, const BwdArgs&, bool, bool, bool, hipStream_t);                    \
   hipError_t name##_d256_padded(int, const BwdArgs&, bool, bool, bool, hipStream_t);                    \
   hipError_t name(int dtype, int head_dim, const BwdArgs& a, bool w, bool b, bool p, hipStream_t s) {   \
-    const bool padded = a.head_dim != head_dim;                                                         \
+    const bool padded = a.head_dim != head_dim || a.head_dim_v != head_dim;                             \
     switch (head_dim) {                                                                                 \
       case 64: return padded ? name##_d64_padded(dtype, a, w, b, p, s) : name##_d64(dtype, a, w, b, p, s);    \
       case 128: return padded ? name##_d128_padded(dtype, a, w, b, p, s) : name##_d128(dtype, a, w, b, p, s); \

@@ -40,7 +40,7 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
   const int row = blockIdx.x * ROWS + tid / LPR;
   const int cc = tid % LPR;
   float acc = 0.f;
-  if (row < si.seqlen_q && cc * 8 < a.head_dim) {   // columns past the tensors' head dim do not exist
+  if (row < si.seqlen_q && cc * 8 < a.head_dim_v) {   // columns past the head dim of Out and dOut do not exist
     const int64_t ro = (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h + (int64_t)(si.q_start + row) * a.so.s;
     const int64_t rd = (int64_t)si.batch_index * a.sdo.z + (int64_t)h * a.sdo.h + (int64_t)(si.q_start + row) * a.sdo.s;
     const op_t o = *reinterpret_cast<const op_t*>(reinterpret_cast<const T*>(a.out) + ro + cc * 8);
@@ -103,7 +103,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int d_act = kPad ? a.head_dim : D;   // <= D, multiple of 8; a constant unless the head dim is rounded up
+  // columns of Q/K/dQ/dK and of V/Out/dOut/dV: <= D, multiples of 8; constants unless a head dim is rounded up
+  const int d_qk = kPad ? a.head_dim : D, d_v = kPad ? a.head_dim_v : D;
 
   const SeqInfo si = get_seq(a.seq, z);
   const int n0 = nt * BN;
@@ -133,10 +134,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          if (32 * db + 8 * g + 4 * hi < d_act) {
-            *reinterpret_cast<q4_t*>(dkptr + 32 * db + 8 * g + 4 * hi) = zero4;
-            *reinterpret_cast<q4_t*>(dvptr + 32 * db + 8 * g + 4 * hi) = zero4;
-          }
+          if (32 * db + 8 * g + 4 * hi < d_qk) *reinterpret_cast<q4_t*>(dkptr + 32 * db + 8 * g + 4 * hi) = zero4;
+          if (32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(dvptr + 32 * db + 8 * g + 4 * hi) = zero4;
         }
     }
     return;
@@ -152,9 +151,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   for (int k = 0; k < KS; ++k) {
     // columns past the tensors' head dim are zero (head dims are rounded up to D)
     const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bool in = 16 * k + 8 * hi < d_act;
-    kreg[k] = in ? *reinterpret_cast<const op_t*>(kptr + 16 * k + 8 * hi) : zero8;
-    vreg[k] = in ? *reinterpret_cast<const op_t*>(vptr + 16 * k + 8 * hi) : zero8;
+    kreg[k] = 16 * k + 8 * hi < d_qk ? *reinterpret_cast<const op_t*>(kptr + 16 * k + 8 * hi) : zero8;
+    vreg[k] = 16 * k + 8 * hi < d_v ? *reinterpret_cast<const op_t*>(vptr + 16 * k + 8 * hi) : zero8;
   }
 
   f32x16 dk[DB], dv[DB];
@@ -184,10 +182,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   op_t qch[CH], doch[CH], och[kInlineDelta ? CH : 1];
   float l_stage = 0.f, d_stage = 0.f;
   const int r0 = tid / LPR, cc0 = tid % LPR;
-  const bool col_ok = cc0 * 8 < d_act;
-  const int q_voff = col_ok ? r0 * (int)a.sq.s * 2 + cc0 * 16 : kVoffOutOfRange,       // bytes inside a tile
-            do_voff = col_ok ? r0 * (int)a.sdo.s * 2 + cc0 * 16 : kVoffOutOfRange,
-            o_voff = col_ok ? r0 * (int)a.so.s * 2 + cc0 * 16 : kVoffOutOfRange;
+  const int q_voff = cc0 * 8 < d_qk ? r0 * (int)a.sq.s * 2 + cc0 * 16 : kVoffOutOfRange,       // bytes inside a tile
+            do_voff = cc0 * 8 < d_v ? r0 * (int)a.sdo.s * 2 + cc0 * 16 : kVoffOutOfRange,
+            o_voff = cc0 * 8 < d_v ? r0 * (int)a.so.s * 2 + cc0 * 16 : kVoffOutOfRange;
   const int q_soff = RPI * (int)a.sq.s * 2, do_soff = RPI * (int)a.sdo.s * 2, o_soff = RPI * (int)a.so.s * 2;
   int lds_off[CH];                                                        // bytes inside a tile
 #pragma unroll
@@ -244,13 +241,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
                                                any && bias_lds ? ((rows - 1) * (int)a.sb_m + cols) * 2 : 0, 0x00020000);
       if (live) bb += (int64_t)BM * a.sb_m;
     }
-    q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + d_act) * 2 : 0,
+    q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0,
                                              0x00020000);
     do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
-                                              any ? ((rows - 1) * (int)a.sdo.s + d_act) * 2 : 0, 0x00020000);
+                                              any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0, 0x00020000);
     if (kInlineDelta)
       o_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ob), 0,
-                                               any ? ((rows - 1) * (int)a.so.s + d_act) * 2 : 0, 0x00020000);
+                                               any ? ((rows - 1) * (int)a.so.s + d_v) * 2 : 0, 0x00020000);
     if (tid < BM) {
       const bool ok = tid < rows;
       l_stage = ok ? lse_b[tid] : 0.f;
@@ -590,10 +587,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
           k4[r] = Tr::cvt(dk[db][4 * g + r] * a.sm_scale);   // bwd_kernel_dk_dv.py:387-389
           v4[r] = Tr::cvt(dv[db][4 * g + r]);
         }
-        if (32 * db + 8 * g + 4 * hi < d_act) {
-          *reinterpret_cast<q4_t*>(dkptr + 32 * db + 8 * g + 4 * hi) = k4;
-          *reinterpret_cast<q4_t*>(dvptr + 32 * db + 8 * g + 4 * hi) = v4;
-        }
+        if (32 * db + 8 * g + 4 * hi < d_qk) *reinterpret_cast<q4_t*>(dkptr + 32 * db + 8 * g + 4 * hi) = k4;
+        if (32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(dvptr + 32 * db + 8 * g + 4 * hi) = v4;
       }
   }
 }
@@ -617,7 +612,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int d_act = kPad ? a.head_dim : D;   // <= D, multiple of 8; a constant unless the head dim is rounded up
+  // columns of Q/K/dQ/dK and of V/Out/dOut/dV: <= D, multiples of 8; constants unless a head dim is rounded up
+  const int d_qk = kPad ? a.head_dim : D, d_v = kPad ? a.head_dim_v : D;
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * BM;
@@ -674,7 +670,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          if (32 * db + 8 * g + 4 * hi < d_act) *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = zero4;
+          if (32 * db + 8 * g + 4 * hi < d_qk) *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = zero4;
     }
     zero_db(0, nkt);
     return;
@@ -689,9 +685,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   for (int k = 0; k < KS; ++k) {
     // columns past the tensors' head dim are zero (head dims are rounded up to D)
     const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bool in = 16 * k + 8 * hi < d_act;
-    qreg[k] = in ? *reinterpret_cast<const op_t*>(qptr + 16 * k + 8 * hi) : zero8;
-    doreg[k] = in ? *reinterpret_cast<const op_t*>(doptr + 16 * k + 8 * hi) : zero8;
+    qreg[k] = 16 * k + 8 * hi < d_qk ? *reinterpret_cast<const op_t*>(qptr + 16 * k + 8 * hi) : zero8;
+    doreg[k] = 16 * k + 8 * hi < d_v ? *reinterpret_cast<const op_t*>(doptr + 16 * k + 8 * hi) : zero8;
   }
   const int64_t lo = lse_offset(si, h, a.hq) + row_c;
   const float l_row = a.lse[lo] * kRcpLn2;               // bwd_kernel_dq.py:305
@@ -702,7 +697,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     float acc = 0.f;
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
-      if (16 * k + 8 * hi >= d_act) continue;
+      if (16 * k + 8 * hi >= d_v) continue;
       const op_t o8 = *reinterpret_cast<const op_t*>(optr + 16 * k + 8 * hi);
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc += (float)o8[e] * (float)doreg[k][e];
@@ -745,9 +740,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   static_assert((BN * D / 8) % NT == 0 && NT % LPR == 0, "threads must cover the tile evenly");
   op_t kch[CH], vch[CH];
   const int r0 = tid / LPR, cc0 = tid % LPR;
-  const bool col_ok = cc0 * 8 < d_act;
-  const int k_voff = col_ok ? r0 * (int)a.sk.s * 2 + cc0 * 16 : kVoffOutOfRange,
-            v_voff = col_ok ? r0 * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
+  const int k_voff = cc0 * 8 < d_qk ? r0 * (int)a.sk.s * 2 + cc0 * 16 : kVoffOutOfRange,
+            v_voff = cc0 * 8 < d_v ? r0 * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
   const int k_soff = RPI * (int)a.sk.s * 2, v_soff = RPI * (int)a.sv.s * 2;
   int lds_off[CH];                                                        // bytes inside a tile
 #pragma unroll
@@ -765,9 +759,9 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     int rows = rows_left < BN ? rows_left : BN;
     rows = live ? rows : 0;
     const bool any = rows > 0;
-    k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, any ? ((rows - 1) * (int)a.sk.s + d_act) * 2 : 0,
+    k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, any ? ((rows - 1) * (int)a.sk.s + d_qk) * 2 : 0,
                                              0x00020000);
-    v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, any ? ((rows - 1) * (int)a.sv.s + d_act) * 2 : 0,
+    v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, any ? ((rows - 1) * (int)a.sv.s + d_v) * 2 : 0,
                                              0x00020000);
     if (live) { kt += k_step; vt += v_step; rows_left -= BN; }
   };
@@ -969,7 +963,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         q4_t t4;
 #pragma unroll
         for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(dq[db][4 * g + r] * a.sm_scale);   // bwd_kernel_dq.py:374-376
-        if (32 * db + 8 * g + 4 * hi < d_act) *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = t4;
+        if (32 * db + 8 * g + 4 * hi < d_qk) *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = t4;
       }
   }
   zero_db(0, br.lo);

@@ -52,7 +52,8 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int d_act = kPad ? a.head_dim : D;   // <= D, multiple of 8; a constant unless the head dim is rounded up
+  // columns of Q/K and of V/Out: <= D, multiples of 8; constants unless a head dim is rounded up
+  const int d_qk = kPad ? a.head_dim : D, d_v = kPad ? a.head_dim_v : D;
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * BM;
@@ -83,7 +84,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          if (32 * db + 8 * g + 4 * hi < d_act) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = zero4;
+          if (32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = zero4;
       if (lse_ptr && hi == 0) lse_ptr[row] = __builtin_inff();
     }
     return;
@@ -97,7 +98,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   for (int ks = 0; ks < KS; ++ks) {
     // columns past the tensors' head dim are zero (head dims are rounded up to D)
     const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    qreg[ks] = 16 * ks + 8 * hi < d_act ? *reinterpret_cast<const op_t*>(qptr + 16 * ks + 8 * hi) : zero8;
+    qreg[ks] = 16 * ks + 8 * hi < d_qk ? *reinterpret_cast<const op_t*>(qptr + 16 * ks + 8 * hi) : zero8;
   }
 
   const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
@@ -126,9 +127,8 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   static_assert(NT % LPR == 0, "threads must cover whole rows");
   op_t kreg[CH], vreg[CH];
   const int r0 = tid / LPR, cc0 = tid % LPR;
-  const bool col_ok = cc0 * 8 < d_act;
-  const int kvoff = col_ok ? r0 * (int)a.sk.s * 2 + cc0 * 16 : kVoffOutOfRange;      // bytes inside a tile
-  const int vvoff = col_ok ? r0 * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
+  const int kvoff = cc0 * 8 < d_qk ? r0 * (int)a.sk.s * 2 + cc0 * 16 : kVoffOutOfRange;      // bytes inside a tile
+  const int vvoff = cc0 * 8 < d_v ? r0 * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
   const int ksoff = RPI * (int)a.sk.s * 2, vsoff = RPI * (int)a.sv.s * 2;
   const int ldsk0 = r0 * KSTR + cc0 * 8, ldsv0 = r0 * VSTR + cc0 * 8;   // elements
 
@@ -141,9 +141,9 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   int rows_left = si.seqlen_k - br.lo * BN;      // > 0
   auto load_next_tile = [&]() {
     const int rows = rows_left < BN ? rows_left : BN;
-    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, (rows - 1) * k_row_bytes + d_act * 2,
+    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, (rows - 1) * k_row_bytes + d_qk * 2,
                                                        0x00020000);
-    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, (rows - 1) * v_row_bytes + d_act * 2,
+    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, (rows - 1) * v_row_bytes + d_v * 2,
                                                        0x00020000);
 #pragma unroll
     for (int i = 0; i < CH; ++i)
@@ -417,7 +417,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
         q4_t t4;
 #pragma unroll
         for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(o[db][4 * g + r] * inv);
-        if (32 * db + 8 * g + 4 * hi < d_act) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
+        if (32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
       }
     if (lse_ptr && hi == 0)
       lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
@@ -484,7 +484,8 @@ hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// kPad: the tensors' head dim (FwdArgs::head_dim) is smaller than D and the excess columns are masked.
+// kPad: a head dim of the tensors (FwdArgs::head_dim, head_dim_v) is smaller than D and the excess
+// columns are masked.
 template <typename T, int D, bool kPad>
 hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t stream) {
   constexpr int BM = FwdTile<D>::NW * 32;

@@ -17,7 +17,9 @@ FUDGE = dict(out=3.0, dq=148.0, dk=48.0, dv=36.0, db=17.0)
 LSE_ATOL = 2e-3
 
 
-def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False, bias_layout='padded'):
+def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False, bias_layout='padded',
+                Dv=None):
+    Dv = D if Dv is None else Dv          # head dim of V, Out and dOut
     g = torch.Generator(device='cpu').manual_seed(seed)
 
     def rn(*shape, scale=1.0):
@@ -26,10 +28,10 @@ def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=Fa
     if bshd:   # storage (B, S, H, D) viewed as (B, H, S, D): non-contiguous head stride
         q = rn(B, Sq, Hq, D).transpose(1, 2)
         k = rn(B, Sk, Hk, D).transpose(1, 2)
-        v = rn(B, Sk, Hk, D).transpose(1, 2)
-        do = rn(B, Sq, Hq, D).transpose(1, 2)
+        v = rn(B, Sk, Hk, Dv).transpose(1, 2)
+        do = rn(B, Sq, Hq, Dv).transpose(1, 2)
     else:
-        q = rn(B, Hq, Sq, D); k = rn(B, Hk, Sk, D); v = rn(B, Hk, Sk, D); do = rn(B, Hq, Sq, D)
+        q = rn(B, Hq, Sq, D); k = rn(B, Hk, Sk, D); v = rn(B, Hk, Sk, Dv); do = rn(B, Hq, Sq, Dv)
     b = None
     if bias:
         if bias_layout == 'padded':

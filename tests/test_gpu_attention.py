@@ -16,12 +16,12 @@ DEV = 'cuda'
 
 
 def _run_case(B, Hq, Hk, Sq, Sk, D, dtype, causal, dropout_p=0.0, bias=False, bshd=False,
-              bwd_backend=-1, sm_scale=None, seed=0, bias_layout='padded'):
+              bwd_backend=-1, sm_scale=None, seed=0, bias_layout='padded', Dv=None):
     from aotriton_amd import flash
     from aotriton_amd.autograd import attention, AttentionExtraArgs
     from oracle import fa_ref
     q, k, v, b, do = make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, DEV, seed=seed, bias=bias, bshd=bshd,
-                                 bias_layout=bias_layout)
+                                 bias_layout=bias_layout, Dv=Dv)
     sm_scale = 1.0 / math.sqrt(D) if sm_scale is None else sm_scale
     ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=bwd_backend)
     qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
@@ -108,6 +108,19 @@ def test_head_dims_rounded_up(D, causal, backend):
 
 def test_head_dim_rounded_up_with_bias_dropout_varlen_strides():
     _run_case(1, 2, 2, 130, 130, 72, torch.float16, (30, 0), dropout_p=0.3, bias=True)
+
+
+@pytest.mark.parametrize('D,Dv', [(192, 128), (128, 64), (64, 128), (40, 72), (96, 256), (256, 8)])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_head_dims_of_qk_and_v_differ(D, Dv, causal, backend):
+    # Q/K with D columns, V/Out/dOut with Dv (hdim_qk != hdim_vo, modules/flash/csrc/attn_fwd.cc:76-82):
+    # both run on the compiled head dim that holds the larger one
+    _run_case(2, 4, 2, 203, 171, D, torch.float16 if D == 40 else torch.bfloat16, causal, bwd_backend=backend, Dv=Dv)
+
+
+def test_head_dims_of_qk_and_v_differ_with_bias_and_dropout():
+    _run_case(1, 2, 1, 140, 150, 192, torch.bfloat16, (40, 3), dropout_p=0.2, bias=True, Dv=128)
 
 
 @pytest.mark.parametrize('causal', [1, 2])

@@ -81,12 +81,13 @@ def test_mk_aotensor_ranks():
     assert flash.cast_dtype(torch.float32) == DType.kFloat32
 
 
-def _fwd_params(D=128, dtype=torch.bfloat16, Hq=4, Hk=2, Sq=64, Sk=80, B=2):
+def _fwd_params(D=128, dtype=torch.bfloat16, Hq=4, Hk=2, Sq=64, Sk=80, B=2, Dv=None):
     """Views over CPU tensors: fine for the pure-host checks (nothing is launched)."""
     from aotriton_amd import flash
     from aotriton_amd.pyaotriton.v3.flash import attn_fwd_params
+    Dv = D if Dv is None else Dv
     keep = dict(q=torch.zeros(B, Hq, Sq, D, dtype=dtype), k=torch.zeros(B, Hk, Sk, D, dtype=dtype),
-                v=torch.zeros(B, Hk, Sk, D, dtype=dtype), o=torch.zeros(B, Hq, Sq, D, dtype=dtype),
+                v=torch.zeros(B, Hk, Sk, Dv, dtype=dtype), o=torch.zeros(B, Hq, Sq, Dv, dtype=dtype),
                 M=torch.zeros(B * Hq, Sq))
     p = attn_fwd_params()
     p.Q = flash.mk_aotensor(keep['q']); p.K = flash.mk_aotensor(keep['k']); p.V = flash.mk_aotensor(keep['v'])
@@ -98,6 +99,7 @@ def _fwd_params(D=128, dtype=torch.bfloat16, Hq=4, Hk=2, Sq=64, Sk=80, B=2):
 def test_validate_fwd_error_contract():
     from aotriton_amd.pyaotriton import hipError_t as E, T4, T2, DType
     from aotriton_amd.pyaotriton.v3.flash import validate_fwd, attn_fwd_params, attn_options, query_fwd_config
+    from aotriton_amd.flash import mk_aotensor as flash_mk
     p, keep = _fwd_params()
     assert validate_fwd(p, attn_fwd_params.kVersion) == E.hipSuccess
     assert validate_fwd(p, 2) == E.hipErrorInvalidSymbol                       # version gate
@@ -105,6 +107,12 @@ def test_validate_fwd_error_contract():
     assert validate_fwd(p2, 3) == E.hipSuccess                                 # rounded up to 128, columns masked
     err, cfg = query_fwd_config(p2)
     assert err == E.hipSuccess and cfg.head_dim == 128
+    p5, k5 = _fwd_params(D=192, Dv=128)                                        # Dqk != Dv: the larger one picks the kernel
+    err, cfg = query_fwd_config(p5)
+    assert err == E.hipSuccess and cfg.head_dim == 256
+    p6, k6 = _fwd_params(D=64, Dv=128)
+    p6.Out = flash_mk(k6['q'])                                                 # Out must have V's head dim
+    assert validate_fwd(p6, 3) == E.hipErrorInvalidValue
     for bad in (512, 100):                                                     # > 256, or rows not a multiple of 16 bytes
         pb, kb = _fwd_params(D=bad)
         assert validate_fwd(pb, 3) == E.hipErrorNotSupported
