@@ -12,14 +12,10 @@ import torch
 from .autograd import attention, AttentionExtraArgs
 
 
-def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False,
-                                 scale=None, enable_gqa=False, extra=None):
-    """Same signature and semantics as torch.nn.functional.scaled_dot_product_attention for
-    4-D fp16/bf16 CUDA tensors (B, H, L, E), with these limits: the head dims (of q/k, and of
-    v) are multiples of 8 up to 256; a boolean mask is turned into an additive one
-    (0 / -inf), and a query row that the mask hides completely yields zeros instead of NaN;
-    dropout uses the operators' Philox stream (seed/offsets in `extra`), not torch's generator.
-    """
+def prepare(query, key, value, attn_mask, is_causal, scale, enable_gqa):
+    """Argument checks and layout fixes shared by the SDPA-shaped entry points: returns
+    (q, k, v, bias, sm_scale) with unit last strides and the mask as an additive
+    (B, H, L, S) bias (None without a mask)."""
     if query.dim() != 4 or key.dim() != 4 or value.dim() != 4:
         raise ValueError('expected (batch, heads, seq, head_dim) tensors')
     if is_causal and attn_mask is not None:
@@ -41,6 +37,18 @@ def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.
         bias = m.expand(q.shape[0], hq, q.shape[2], k.shape[2])
         if bias.stride(-1) != 1:
             bias = bias.contiguous()
+    return q, k, v, bias, sm_scale
+
+
+def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False,
+                                 scale=None, enable_gqa=False, extra=None):
+    """Same signature and semantics as torch.nn.functional.scaled_dot_product_attention for
+    4-D fp16/bf16 CUDA tensors (B, H, L, E), with these limits: the head dims (of q/k, and of
+    v) are multiples of 8 up to 256; a boolean mask is turned into an additive one
+    (0 / -inf), and a query row that the mask hides completely yields zeros instead of NaN;
+    dropout uses the operators' Philox stream (seed/offsets in `extra`), not torch's generator.
+    """
+    q, k, v, bias, sm_scale = prepare(query, key, value, attn_mask, is_causal, scale, enable_gqa)
     out, _, _ = attention(q, k, v, bias, bool(is_causal), sm_scale, float(dropout_p),
                           extra or AttentionExtraArgs())
     return out
