@@ -254,3 +254,102 @@ def test_padded_and_strided_varlen(layout, causal, backend):
         assert torch.isnan(o[1, :, lens[1]:]).all() and torch.isnan(dk[1, :, lens[1]:]).all()
     else:
         assert torch.isnan(o[:, :, lens[0]:starts[1]]).all() and torch.isnan(dv[:, :, lens[0]:starts[1]]).all()
+
+
+def test_config4_full_size_properties():
+    """GQA varlen at full size: Hq 32, Hkv 8, D 128 bf16 causal, 16 packed sequences of
+    256..8192 tokens (~68K in all).  Checked per sequence, so at any size: (1) the first
+    row of a sequence attends to its first key only; (2) the shortest and the longest
+    sequence match the dense oracle for one kv-head and its four q-heads; (3) the keys'
+    dV sums equal the dO sums of the q-heads that share the kv-head."""
+    from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
+    from oracle import fa_ref
+    rng = np.random.default_rng(1234)
+    lens = rng.integers(256, 8193, size=16)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    T = int(cu[-1])
+    Hq, Hk, D = 32, 8, 128
+    dt = torch.bfloat16
+    g = torch.Generator(device=DEV).manual_seed(4)
+    mk = lambda H: torch.randn(1, T, H, D, device=DEV, generator=g).to(dt).transpose(1, 2)
+    q, k, v, do = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+    sm = 1.0 / math.sqrt(D)
+    TL = -2147483647
+    for backend in (0, 1):
+        qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+        o, _, L = attention_varlen(qg, kg, vg, lens, lens, True, sm, 0.0,
+                                   AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend))
+        o.backward(do)
+        torch.cuda.synchronize()
+        for t in (o, L, qg.grad, kg.grad, vg.grad):
+            assert torch.isfinite(t).all()
+        first = torch.from_numpy(cu[:-1]).to(DEV)
+        assert torch.equal(o[0, :, first], v[0, :, first].repeat_interleave(Hq // Hk, dim=0))
+        s00 = (q[0, :, first].float() * k[0, :, first].float().repeat_interleave(Hq // Hk, dim=0)).sum(-1) * sm
+        assert torch.allclose(L[:, first], s00, atol=1e-4, rtol=1e-5)
+        hk = 5
+        hs = slice(hk * 4, hk * 4 + 4)
+        for i in (int(np.argmin(lens)), int(np.argmax(lens))):
+            a, b = int(cu[i]), int(cu[i + 1])
+            qs, ks, vs, dos = q[:, hs, a:b], k[:, hk:hk + 1, a:b], v[:, hk:hk + 1, a:b], do[:, hs, a:b]
+            ro, rl, _ = fa_ref.attn_fwd_ref(qs.float(), ks.float(), vs.float(), None, sm, 3, TL, TL)
+            lo, ll, _ = fa_ref.attn_fwd_ref(qs, ks, vs, None, sm, 3, TL, TL)
+            check('out', o[:, hs, a:b], ro, lo, FUDGE['out'])
+            assert (L[hs, a:b] - rl[0]).abs().max().item() <= LSE_ATOL
+            rg = fa_ref.attn_bwd_ref(qs.float(), ks.float(), vs.float(), None, sm, ro, dos.float(), rl, 3, TL, TL)
+            lg = fa_ref.attn_bwd_ref(qs, ks, vs, None, sm, lo, dos, ll.to(dt), 3, TL, TL)
+            check('dq', qg.grad[:, hs, a:b], rg[0], lg[0], FUDGE['dq'])
+            check('dk', kg.grad[:, hk:hk + 1, a:b], rg[1], lg[1], FUDGE['dk'])
+            check('dv', vg.grad[:, hk:hk + 1, a:b], rg[2], lg[2], FUDGE['dv'])
+        for i in range(len(lens)):
+            a, b = int(cu[i]), int(cu[i + 1])
+            colsum = vg.grad[0, :, a:b].float().sum(dim=1)                            # (Hk, D)
+            dosum = do[0, :, a:b].float().sum(dim=1).view(Hk, Hq // Hk, D).sum(dim=1)
+            assert (colsum - dosum).abs().max().item() < 1.0, (i, (colsum - dosum).abs().max().item())
+
+
+def test_config5_full_size_properties():
+    """Window (1024, 0) + bias + dropout 0.1 (seed 0x1234, offset 0) at B2 H16 S8192 D256
+    fp16: a sampled (batch, head) against the dense oracle with the oracle's own keep
+    mask, dB exactly zero outside the band, everything finite."""
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref, philox
+    B, H, S, D = 2, 16, 8192, 256
+    dt = torch.float16
+    g = torch.Generator(device=DEV).manual_seed(0)
+    rn = lambda *s, sc=1.0: (torch.randn(*s, device=DEV, dtype=torch.float32, generator=g) * sc).to(dt)
+    q, k, v, do = rn(B, H, S, D), rn(B, H, S, D), rn(B, H, S, D), rn(B, H, S, D)
+    bias = torch.empty(B, H, S, S, device=DEV, dtype=dt)
+    for i in range(B):
+        for h in range(H):
+            bias[i, h] = rn(S, S, sc=0.5)
+    sm = 1.0 / math.sqrt(D)
+    p = 0.1
+    qg, kg, vg, bg = [t.requires_grad_() for t in (q, k, v, bias)]
+    ext = AttentionExtraArgs(return_logsumexp=True, philox_seed=0x1234, philox_offset1=0, philox_offset2=0)
+    o, _, L = attention(qg, kg, vg, bg, (1024, 0), sm, p, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    for t in (o, L, qg.grad, kg.grad, vg.grad):
+        assert torch.isfinite(t).all()
+    bsel, hsel = 1, 7
+    sl = lambda t: t.detach()[bsel:bsel + 1, hsel:hsel + 1]
+    keep = torch.from_numpy(philox.dropout_keep_mask(B, H, S, S, p, 0x1234, 0, b_sel=[bsel], h_sel=[hsel])).to(DEV)
+    f = lambda t: sl(t).float()
+    ro, rl, _ = fa_ref.attn_fwd_ref(f(q), f(k), f(v), f(bias), sm, 3, 1024, 0, p, keep)
+    lo, ll, _ = fa_ref.attn_fwd_ref(sl(q), sl(k), sl(v), sl(bias), sm, 3, 1024, 0, p, keep)
+    check('out', sl(o), ro, lo, FUDGE['out'])
+    assert (L.view(B, H, S)[bsel, hsel] - rl[0, 0]).abs().max().item() <= LSE_ATOL
+    rg = fa_ref.attn_bwd_ref(f(q), f(k), f(v), f(bias), sm, ro, f(do), rl, 3, 1024, 0, p, keep)
+    lg = fa_ref.attn_bwd_ref(sl(q), sl(k), sl(v), sl(bias), sm, lo, sl(do), ll.to(dt), 3, 1024, 0, p, keep)
+    check('dq', sl(qg.grad), rg[0], lg[0], FUDGE['dq'])
+    check('dk', sl(kg.grad), rg[1], lg[1], FUDGE['dk'])
+    check('dv', sl(vg.grad), rg[2], lg[2], FUDGE['dv'])
+    check('db', sl(bg.grad), rg[3], lg[3], FUDGE['db'])
+    # outside the band dB is exactly zero, for every (batch, head)
+    m = torch.arange(S, device=DEV).view(S, 1)
+    n = torch.arange(S, device=DEV).view(1, S)
+    outside = (n > m) | (n < m - 1024)
+    for i in range(B):
+        for h in range(0, H, 5):
+            assert not bg.grad[i, h][outside].any()
