@@ -128,3 +128,43 @@ def test_sdpa_dropout_follows_torch_generator():
     keep = torch.from_numpy(philox.dropout_keep_mask(B, H, Sq, Sk, 0.3, 11, 0)).to(DEV)
     ro, _, _ = fa_ref.attn_fwd_ref(q.float(), k.float(), v.float(), None, 1.0 / 8, 0, 0, 0, 0.3, keep)
     assert (a.float() - ro).abs().max().item() < 0.05
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dropout_p', [0.0, 0.2])
+def test_forward_and_backward_replay_from_a_hip_graph(dropout_p):
+    """The operators allocate nothing themselves and launch on the caller's stream, so a
+    forward + backward can be captured into a graph.  Every replay (with eager work and
+    synchronisation between replays) must reproduce the eager result bit for bit."""
+    from aotriton_amd import torch_ops  # noqa: F401
+    q, k, v, _, do = _inputs(B=2, Hq=4, Hk=2, Sq=300, Sk=300, D=128, seed=9)
+    sm = 1.0 / math.sqrt(128)
+    seed, off = _u64(0x5EED), _u64(64)
+    args = (dropout_p, 3, -2147483647, -2147483647, sm, seed, off)
+
+    def run():
+        o, lse = torch.ops.aotriton_amd.flash_attention_forward(q, k, v, None, *args)
+        dq, dk, dv, _ = torch.ops.aotriton_amd.flash_attention_backward(do, q, k, v, None, o, lse, *args, False, -1)
+        return o, lse, dq, dk, dv
+
+    eager = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()                                   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for rep in range(3):
+        for t in captured:
+            t.fill_(float('nan'))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, e, c in zip(('out', 'lse', 'dq', 'dk', 'dv'), eager, captured):
+            assert torch.equal(e, c), f'replay {rep}: {name} differs from the eager run'
+        again = run()                           # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(again[0], eager[0])
