@@ -67,7 +67,11 @@ struct DkDvSmem {   // per stage: Q, dO (swizzled, one copy each); L, delta; bia
   static constexpr int BIAS_BYTES = BM * BIAS_STR;
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * BM * 4 + BIAS_BYTES;
   static constexpr int STAGES = 2;
-  static constexpr int BYTES = STAGES * STAGE_BYTES;
+  // D = 256: the registers cannot hold both K and V of the wave's keys next to the dK and dV
+  // accumulators, so the workgroup's V tile (128 keys) stays in LDS for the whole item
+  static constexpr int V_OFF = STAGES * STAGE_BYTES;
+  static constexpr int V_BYTES = D >= 256 ? 128 * D * 2 : 0;
+  static constexpr int BYTES = V_OFF + V_BYTES;
 };
 
 template <int D, int BN>
@@ -146,13 +150,14 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
                   (int64_t)(si.k_start + key_c) * a.sk.s;
   const T* vptr = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                   (int64_t)(si.k_start + key_c) * a.sv.s;
-  op_t kreg[KS], vreg[KS];
+  constexpr bool kVLds = SM::V_BYTES > 0;       // V operands come from LDS instead of registers
+  op_t kreg[KS], vreg[kVLds ? 1 : KS];
 #pragma unroll
   for (int k = 0; k < KS; ++k) {
     // columns past the tensors' head dim are zero (head dims are rounded up to D)
     const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     kreg[k] = 16 * k + 8 * hi < d_qk ? *reinterpret_cast<const op_t*>(kptr + 16 * k + 8 * hi) : zero8;
-    vreg[k] = 16 * k + 8 * hi < d_v ? *reinterpret_cast<const op_t*>(vptr + 16 * k + 8 * hi) : zero8;
+    if (!kVLds) vreg[k] = 16 * k + 8 * hi < d_v ? *reinterpret_cast<const op_t*>(vptr + 16 * k + 8 * hi) : zero8;
   }
 
   f32x16 dk[DB], dv[DB];
@@ -390,6 +395,12 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     }
     // row statistics of the tile's queries and the first dO operands
     l4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ls, 0));
+    const char* Vt = smem_raw + SM::V_OFF;
+    op_t vl[3];          // ring of V operands when they come from LDS
+    if (kVLds) {
+      vl[0] = swz_read_row<T, D>(Vt, row_a, 0, wave);
+      vl[1] = swz_read_row<T, D>(Vt, row_a, 1, wave);
+    }
 #pragma unroll
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
@@ -464,9 +475,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         for (int mb = 0; mb < MB; ++mb)
           xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(dOb, row_a, k + kAhead, mb);
       }
+      if (kVLds && k + 2 < KS) vl[(k + 2) % 3] = swz_read_row<T, D>(Vt, row_a, k + 2, wave);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], vreg[k], k == 0 ? zero16 : dp[mb]);
+        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kVLds ? vl[k % 3] : vreg[kVLds ? 0 : k], k == 0 ? zero16 : dp[mb]);
         const int gidx = k * MB + mb;
         if (EPG1 >= 1) {
 #pragma unroll
@@ -489,9 +501,19 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     }
     // delta of the tile's queries, first transposed dO operands
     d4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 0));
-    op_t ta[2][DB];
+    // Transposed operands are read ahead of their MFMAs: a whole 16-query step ahead, or,
+    // where that would take too many registers (D = 256), through a ring of kRing operands.
+    constexpr bool kRingTa = DB >= 8;
+    constexpr int kRing = 4;
+    op_t ta[kRingTa ? 1 : 2][kRingTa ? kRing : DB];
+    auto ta_read = [&](const char* tile, int gidx) { return swz_read_tr<T, D>(tile, tr_a0, tr_a1, gidx / DB, gidx % DB); };
+    if (kRingTa) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, 0, db);
+      for (int gi = 0; gi < kRing - 1; ++gi) ta[0][gi] = ta_read(dOb, gi);
+    } else {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, 0, db);
+    }
 
     // ---- dV^T += dO^T P, with ds behind its MFMAs --------------------------------
     constexpr int G3 = TS * DB;
@@ -501,9 +523,14 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     for (int t = 0; t < TS; ++t) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        if (t + 1 < TS) ta[(t + 1) & 1][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, t + 1, db);
-        dv[db] = Tr::mfma(ta[t & 1][db], pb[t], dv[db]);
         const int gidx = t * DB + db;
+        if (kRingTa) {
+          if (gidx + kRing - 1 < TS * DB) ta[0][(gidx + kRing - 1) % kRing] = ta_read(dOb, gidx + kRing - 1);
+          dv[db] = Tr::mfma(ta[0][gidx % kRing], pb[t], dv[db]);
+        } else {
+          if (t + 1 < TS) ta[(t + 1) & 1 & (kRingTa ? 0 : 1)][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, t + 1, db);
+          dv[db] = Tr::mfma(ta[t & 1 & (kRingTa ? 0 : 1)][db], pb[t], dv[db]);
+        }
         if (EPG3 >= 1) {
 #pragma unroll
           for (int e = 0; e < (EPG3 >= 1 ? EPG3 : 1); ++e) {
@@ -523,18 +550,29 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       }
     }
     // ---- dK^T += Q^T dS ----------------------------------------------------------
+    if (kRingTa) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, 0, db);
+      for (int gi = 0; gi < kRing - 1; ++gi) ta[0][gi] = ta_read(Qb, gi);
+    } else {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, 0, db);
+    }
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
-      if (t + 1 < TS) {
+      if (!kRingTa && t + 1 < TS) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          ta[(t + 1) & 1][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, t + 1, db);
+          ta[(t + 1) & 1 & (kRingTa ? 0 : 1)][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, t + 1, db);
       }
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        dk[db] = Tr::mfma(ta[t & 1][db], sb[t], dk[db]);
+        if (kRingTa) {
+          const int gidx = t * DB + db;
+          if (gidx + kRing - 1 < TS * DB) ta[0][(gidx + kRing - 1) % kRing] = ta_read(Qb, gidx + kRing - 1);
+          dk[db] = Tr::mfma(ta[0][gidx % kRing], sb[t], dk[db]);
+        } else {
+          dk[db] = Tr::mfma(ta[t & 1 & (kRingTa ? 0 : 1)][db], sb[t], dk[db]);
+        }
         // the next tile's LDS writes ride behind these MFMAs
         constexpr int per = (STORE_PIECES + G4 - 1) / G4;
 #pragma unroll
@@ -548,6 +586,22 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     store_stats(stage ^ 1);
   };
 
+  if (kVLds) {
+    // the workgroup's V tile, rows past the sequence and columns past the head dim zero
+    const T* vt = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
+                  (int64_t)(si.k_start + n0) * a.sv.s;
+    const int rows = si.seqlen_k - n0 < BN ? si.seqlen_k - n0 : BN;
+    const auto v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0,
+                                                        ((rows - 1) * (int)a.sv.s + d_v) * 2, 0x00020000);
+    constexpr int VCH = BN * D / 8 / NT;
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int row = r0 + i * RPI;
+      const int voff = cc0 * 8 < d_v ? row * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
+      const op_t x = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(v_rs, voff, 0, 0));
+      *reinterpret_cast<op_t*>(smem_raw + SM::V_OFF + Swz<D>::addr(row, cc0)) = x;
+    }
+  }
   fetch_begin(true, 0, 0);
 #pragma unroll
   for (int i = 0; i < FETCH_PIECES; ++i) fetch_piece(i);
