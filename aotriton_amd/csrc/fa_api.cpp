@@ -103,7 +103,6 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   const int dtype = Q.dtype;
   if (dtype != FA_DTYPE_FLOAT16 && dtype != FA_DTYPE_BFLOAT16 && dtype != FA_DTYPE_FLOAT32)
     return FA_ERROR_INVALID_VALUE;
-  if (!is_16bit(dtype)) return FA_ERROR_NOT_SUPPORTED;   // fp32 kernels are not built
   int e;
   if ((e = check_act(Q, dtype)) != FA_SUCCESS) return e;
   if ((e = check_act(K, dtype)) != FA_SUCCESS) return e;
@@ -240,8 +239,15 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
     for (int i = 0; i < 4; ++i)
       if (p->DB.sizes[i] != p->B.sizes[i]) return FA_ERROR_INVALID_VALUE;
   }
-  const int be = bwd_backend(p, opt);
+  int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2
+  if (be == 1 && !is_16bit(dt)) {
+    // fp32 has the split kernels only: a forced fused backend cannot take the input, an
+    // unforced choice falls back to split when a delta buffer is there (template/op.cc:57-70)
+    const bool forced = opt != nullptr && opt->force_backend_index >= 0;
+    if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
+    be = 0;
+  }
   if (be == 0) {
     if (p->D.eager.ptr == nullptr && p->D.acquire == nullptr) return FA_ERROR_INVALID_VALUE;
     if (p->D.eager.ptr != nullptr && p->D.eager.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
@@ -252,6 +258,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
+  if (dtype == FA_DTYPE_FLOAT32) return fa::run_fwd_f32(d, a, stream);
   const bool padded = a.head_dim != d || a.head_dim_v != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
     case 64: return (padded ? fa::run_fwd_d64_padded : fa::run_fwd_d64)(dtype, a, s.windowed, s.bias, s.dropout, stream);
@@ -498,11 +505,13 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
       acquired = true;
     }
     a.delta = static_cast<float*>(delta.ptr);
-    if (kernel_slot < 0 || kernel_slot == 0) err = fa::run_bwd_preprocess(dt, s.d, a, stream);
+    const bool f32 = dt == FA_DTYPE_FLOAT32;
+    if (kernel_slot < 0 || kernel_slot == 0)
+      err = f32 ? fa::run_bwd_f32(s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
     if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 1))
-      err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      err = f32 ? fa::run_bwd_f32(s.d, 1, a, stream) : fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 2))
-      err = fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      err = f32 ? fa::run_bwd_f32(s.d, 2, a, stream) : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);   // attn_bwd.cc:157
   } else {
     a.delta = nullptr;

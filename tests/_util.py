@@ -1,7 +1,8 @@
 """Shared helpers for the GPU parity tests: seeded inputs and the reference's
 tolerance model (modules/flash/tests/_common_test.py:459-495):
     max|out - ref_hp| <= max(1e-5, fudge * max|ref_hp - ref_lp|)
-with ref_hp the oracle in fp32 and ref_lp the oracle in the input dtype.
+with ref_hp the oracle in fp32 and ref_lp the oracle in the input dtype (fp64 and fp32
+for fp32 inputs, _common_test.py:347).
 Fudge factors: out 3.0, dq 148, dk 48, dv 36, db 17 (_common_test.py:171-180,384-407).
 """
 import math
@@ -54,7 +55,7 @@ def ref_fwd(q, k, v, b, sm_scale, ct, wl, wr, p, keep, dtype):
 
 
 def check(name, out, ref_hp, ref_lp, fudge, mask=None):
-    out = out.float(); ref_hp = ref_hp.float(); ref_lp = ref_lp.float()
+    out = out.double(); ref_hp = ref_hp.double(); ref_lp = ref_lp.double()
     if mask is not None:
         out = out[mask]; ref_hp = ref_hp[mask]; ref_lp = ref_lp[mask]
     assert not torch.isnan(out).any(), f'{name}: NaN in output'

@@ -34,7 +34,8 @@ def _run_case(B, Hq, Hk, Sq, Sk, D, dtype, causal, dropout_p=0.0, bias=False, bs
     ct, wl, wr = flash.translate_causal(causal)
     keep = keep_mask_from_oracle(B, Hq, Sq, Sk, dropout_p, ext.philox_seed,
                                  ext.philox_offset1 + ext.philox_offset2, DEV)
-    f32 = lambda t: None if t is None else t.float()
+    hp = torch.float64 if dtype == torch.float32 else torch.float32      # _common_test.py:347
+    f32 = lambda t: None if t is None else t.to(hp)
     ro, rl, _ = fa_ref.attn_fwd_ref(f32(q), f32(k), f32(v), f32(b), sm_scale, ct, wl, wr, dropout_p, keep)
     lo, ll, _ = fa_ref.attn_fwd_ref(q, k, v, b, sm_scale, ct, wl, wr, dropout_p, keep)
     live = torch.isfinite(rl)
@@ -121,6 +122,33 @@ def test_head_dims_of_qk_and_v_differ(D, Dv, causal, backend):
 
 def test_head_dims_of_qk_and_v_differ_with_bias_and_dropout():
     _run_case(1, 2, 1, 140, 150, 192, torch.bfloat16, (40, 3), dropout_p=0.2, bias=True, Dv=128)
+
+
+def test_fp32_baseline_config_1():
+    # B2 H4 S128 D64 fp32 non-causal: the reference's CPU-runnable configuration, on the GPU
+    _run_case(2, 4, 4, 128, 128, 64, torch.float32, False, sm_scale=1.0 / 8)
+
+
+@pytest.mark.parametrize('case', [
+    dict(D=64, causal=True), dict(D=128, causal=(13, 4), Hk=2, sq=203, sk=171, bshd=True),
+    dict(D=256, causal=2, sq=90, sk=150), dict(D=128, causal=True, bias=True, dropout_p=0.25, sq=150, sk=150),
+    dict(D=40, causal=False, Dv=72, Hk=1, sq=77, sk=129), dict(D=128, causal=1, sq=300, sk=140),
+])
+def test_fp32_inputs(case):
+    # fp32 tensors run on the vector-ALU kernels; the oracle is fp64 against fp32
+    c = dict(Hk=4, sq=128, sk=128, bias=False, dropout_p=0.0, bshd=False, Dv=None)
+    c.update(case)
+    _run_case(2, 4, c['Hk'], c['sq'], c['sk'], c['D'], torch.float32, c['causal'], dropout_p=c['dropout_p'],
+              bias=c['bias'], bshd=c['bshd'], Dv=c['Dv'], bwd_backend=0)
+
+
+def test_fp32_has_no_fused_backend():
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    q, k, v, _, do = make_inputs(1, 2, 2, 64, 64, 64, torch.float32, DEV)
+    qg = q.clone().requires_grad_()
+    o, _, _ = attention(qg, k, v, None, False, 0.125, 0.0, AttentionExtraArgs(bwd_backend=1))
+    with pytest.raises(NotImplementedError):      # hipErrorPeerAccessUnsupported: the backend cannot take the input
+        o.backward(do)
 
 
 @pytest.mark.parametrize('causal', [1, 2])

@@ -55,6 +55,37 @@ def test_compact_varlen_gqa(dtype, D, causal, backend):
     check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
 
 
+def test_compact_varlen_fp32():
+    # packed sequences through the fp32 kernels; oracle in fp64 against fp32
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
+    from oracle import fa_ref
+    lens = np.array([5, 64, 131, 17])
+    T = int(lens.sum())
+    Hq, Hk, D = 4, 2, 64
+    cu = [0] + np.cumsum(lens).tolist()
+    g = torch.Generator().manual_seed(6)
+    mk = lambda H: torch.randn(1, T, H, D, generator=g).to(DEV).transpose(1, 2)
+    q, k, v, do = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+    sm = 1.0 / math.sqrt(D)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    o, _, L = attention_varlen(qg, kg, vg, lens, lens, True, sm, 0.0,
+                               AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=0))
+    o.backward(do)
+    torch.cuda.synchronize()
+    ct, wl, wr = flash.translate_causal(True)
+    f = lambda t: t.double()
+    ro, rl = fa_ref.varlen_fwd_ref(f(q), f(k), f(v), cu, cu, sm, ct, wl, wr)
+    lo, ll = fa_ref.varlen_fwd_ref(q, k, v, cu, cu, sm, ct, wl, wr)
+    check('out', o, ro, lo, FUDGE['out'])
+    assert (L - rl).abs().max().item() <= LSE_ATOL
+    rg = fa_ref.varlen_bwd_ref(f(q), f(k), f(v), cu, cu, sm, ro, f(do), rl, ct, wl, wr)
+    lg = fa_ref.varlen_bwd_ref(q, k, v, cu, cu, sm, lo, do, ll, ct, wl, wr)
+    check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
+    check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
+    check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
+
+
 def test_varlen_dropout_mask_uses_sequence_index_and_max_seqlens():
     from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
     from oracle import fa_ref, philox
