@@ -119,11 +119,11 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   // Head dims are rounded up to a compiled one and the excess columns are masked in
   // the kernels (PADDED_HEAD, attn_fwd.cc:76-82,109); 16-byte granularity.  Dqk and Dv
   // may differ: both run on the compiled head dim that holds the larger one.
-  if (dqk <= 0 || dqk > 256 || dqk % 8 != 0 || dv <= 0 || dv > 256 || dv % 8 != 0) return FA_ERROR_NOT_SUPPORTED;
+  if (dqk <= 0 || dqk > 512 || dqk % 8 != 0 || dv <= 0 || dv > 512 || dv % 8 != 0) return FA_ERROR_NOT_SUPPORTED;
   s.d_qk = dqk;
   s.d_v = dv;
   const int dmax = dqk > dv ? dqk : dv;
-  s.d = dmax <= 64 ? 64 : (dmax <= 128 ? 128 : 256);
+  s.d = dmax <= 64 ? 64 : (dmax <= 128 ? 128 : (dmax <= 256 ? 256 : 512));   // 512: vector-ALU kernels
   s.max_sq = (int)Q.sizes[2];
   s.max_sk = (int)K.sizes[2];
   s.num_seqlens = 0;
@@ -241,8 +241,8 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   }
   int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2
-  if (be == 1 && !is_16bit(dt)) {
-    // fp32 has the split kernels only: a forced fused backend cannot take the input, an
+  if (be == 1 && (!is_16bit(dt) || s.d > 256)) {
+    // the vector-ALU kernels (fp32, head dims above 256) exist for the split backend only: a forced fused backend cannot take the input, an
     // unforced choice falls back to split when a delta buffer is there (template/op.cc:57-70)
     const bool forced = opt != nullptr && opt->force_backend_index >= 0;
     if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
@@ -258,7 +258,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
-  if (dtype == FA_DTYPE_FLOAT32) return fa::run_fwd_f32(d, a, stream);
+  if (dtype == FA_DTYPE_FLOAT32 || d > 256) return fa::run_fwd_valu(dtype, d, a, stream);
   const bool padded = a.head_dim != d || a.head_dim_v != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
     case 64: return (padded ? fa::run_fwd_d64_padded : fa::run_fwd_d64)(dtype, a, s.windowed, s.bias, s.dropout, stream);
@@ -333,10 +333,15 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   Shape s{};
   int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
   if (e != FA_SUCCESS) return e;
-  const fa::TileShape t = fa::fwd_tile_shape(s.d);
+  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
+  const fa::TileShape t = valu ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(s.d);
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
-  {
+  if (valu) {
+    out->grid[0] = (s.max_sq + 31) / 32;
+    out->grid[1] = s.hq;
+    out->grid[2] = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+  } else {
     const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
     const int zh_per_xcd = (nz * s.hq + fa::kNumXcd - 1) / fa::kNumXcd;
     const int ratio = s.hq / s.hk;
@@ -363,7 +368,10 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   int be = 0;
   int e = validate_bwd(params, FA_BWD_PARAMS_VERSION, options, &s, &be);
   if (e != FA_SUCCESS) return e;
-  const fa::TileShape t = fa::bwd_tile_shape(s.d, kernel_slot);
+  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
+  if (valu && kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
+  const fa::TileShape t = valu ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
+                               : fa::bwd_tile_shape(s.d, kernel_slot);
   const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
@@ -376,7 +384,11 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   const int ratio = s.hq / s.hk;
   out->grid[1] = 1;
   out->grid[2] = 1;
-  switch (kernel_slot) {
+  if (valu) {
+    out->grid[0] = kernel_slot == 1 ? nt : mt;
+    out->grid[1] = kernel_slot == 1 ? s.hk : s.hq;
+    out->grid[2] = nz;
+  } else switch (kernel_slot) {
     case 0: out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz; break;
     case 1: out->grid[0] = grid1d(s.hk, 2, nt); break;
     case 2: out->grid[0] = grid1d(s.hq, ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2, mt); break;
@@ -437,7 +449,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
   a.atomic_counter = static_cast<int32_t*>(p->persistent_atomic_counter.ptr);
   a.num_cu = dev->num_cu;
 
-  const fa::TileShape t = fa::fwd_tile_shape(s.d);
+  const fa::TileShape t = (p->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256) ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(s.d);
   FA_LOG(4, "attn_fwd: D=%d BLOCK_M=%d BLOCK_N=%d waves=%d lds=%d windowed=%d bias=%d dropout=%d nseq=%d",
          s.d, t.block_m, t.block_n, t.num_waves, t.lds_bytes, (int)s.windowed, (int)s.bias,
          (int)s.dropout, s.num_seqlens);
@@ -505,13 +517,13 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
       acquired = true;
     }
     a.delta = static_cast<float*>(delta.ptr);
-    const bool f32 = dt == FA_DTYPE_FLOAT32;
+    const bool f32 = dt == FA_DTYPE_FLOAT32 || s.d > 256;      // vector-ALU kernels
     if (kernel_slot < 0 || kernel_slot == 0)
-      err = f32 ? fa::run_bwd_f32(s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
+      err = f32 ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
     if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 1))
-      err = f32 ? fa::run_bwd_f32(s.d, 1, a, stream) : fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      err = f32 ? fa::run_bwd_valu(dt, s.d, 1, a, stream) : fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 2))
-      err = f32 ? fa::run_bwd_f32(s.d, 2, a, stream) : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      err = f32 ? fa::run_bwd_valu(dt, s.d, 2, a, stream) : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);   // attn_bwd.cc:157
   } else {
     a.delta = nullptr;

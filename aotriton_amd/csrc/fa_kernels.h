@@ -28,9 +28,10 @@ hipError_t run_bwd_dq(int dtype, int head_dim, const BwdArgs& a, bool windowed, 
 hipError_t run_bwd_fused(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 TileShape bwd_tile_shape(int head_dim, int kernel_slot);
 
-// fp32 tensors: vector-ALU kernels (no fp32 MFMA path); head_dim is the compiled one.
-// kernel_slot of the backward: 0 delta, 1 dK/dV, 2 dQ and dB.
-hipError_t run_fwd_f32(int head_dim, const FwdArgs& a, hipStream_t s);
-hipError_t run_bwd_f32(int head_dim, int kernel_slot, const BwdArgs& a, hipStream_t s);
+// Vector-ALU kernels (no MFMA): fp32 tensors at any head dim, every type at head dim 512.
+// head_dim is the compiled one (64, 128, 256, 512).  kernel_slot of the backward: 0 delta,
+// 1 dK/dV, 2 dQ and dB.
+hipError_t run_fwd_valu(int dtype, int head_dim, const FwdArgs& a, hipStream_t s);
+hipError_t run_bwd_valu(int dtype, int head_dim, int kernel_slot, const BwdArgs& a, hipStream_t s);
 
 }  // namespace fa

@@ -1,9 +1,11 @@
-// fp32 inputs: plain vector-ALU kernels, one row of Q (or of K) per group of 8 lanes.
+// Plain vector-ALU kernels, one row of Q (or of K) per group of 8 lanes: the functional path
+// for what the MFMA kernels do not cover, i.e. fp32 tensors (any head dim) and head dims
+// above 256 up to 512 (any type).
 //
-// The reference compiles its Triton kernels for fp32 as well (modules/flash/aot/_common.py
-// lists '*fp32:16' among the tensor types); fp32 is the functional path there too, far
-// from the throughput of the 16-bit MFMA kernels.  These kernels compute exactly what the
-// 16-bit ones do, in the same base-2 formulation
+// The reference compiles its Triton kernels for fp32 and for head dim 512 as well
+// (modules/flash/aot/_common.py:10-14 lists the head dims, '*fp32:16' is among the tensor
+// types).  These kernels compute what the MFMA kernels do, in the same base-2 formulation,
+// with all arithmetic in fp32
 //   forward   modules/flash/kernel/fwd_kernel.py:83-644, fwd_kernel_inner.py:46-287
 //   delta     modules/flash/kernel/bwd_preprocess.py:28-250
 //   dK, dV    modules/flash/kernel/bwd_kernel_dk_dv.py:48-417, bwd_inner_dk_dv.py:28-267
@@ -26,29 +28,43 @@ struct Row {
   float x[DPL];
 };
 
-// columns [0, cols) of a row of D = 8*DPL floats; the rest reads as zero
-template <int DPL>
-__device__ __forceinline__ Row<DPL> load_row(const float* p, int sub, int cols, bool ok) {
+// four consecutive elements of the tensors' type
+template <typename T> struct Quad { using type = typename Traits<T>::q4_t; };
+template <> struct Quad<float> { using type = f32x4; };
+template <typename T> __device__ __forceinline__ T from_float(float x) { return Traits<T>::cvt(x); }
+template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
+
+// columns [0, cols) of a row of D = 8*DPL elements as floats; the rest reads as zero
+template <int DPL, typename T>
+__device__ __forceinline__ Row<DPL> load_row(const T* p, int sub, int cols, bool ok) {
+  using quad = typename Quad<T>::type;
   Row<DPL> r;
 #pragma unroll
   for (int j = 0; j < DPL / 4; ++j) {
     const int c = 4 * sub + 32 * j;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (ok && c < cols) v = *reinterpret_cast<const f32x4*>(p + c);
+    if (ok && c < cols) {
+      const quad v = *reinterpret_cast<const quad*>(p + c);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) r.x[4 * j + e] = v[e];
+      for (int e = 0; e < 4; ++e) r.x[4 * j + e] = (float)v[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r.x[4 * j + e] = 0.f;
+    }
   }
   return r;
 }
 
-template <int DPL>
-__device__ __forceinline__ void store_row(float* p, const Row<DPL>& r, int sub, int cols, float scale) {
+template <int DPL, typename T>
+__device__ __forceinline__ void store_row(T* p, const Row<DPL>& r, int sub, int cols, float scale) {
+  using quad = typename Quad<T>::type;
 #pragma unroll
   for (int j = 0; j < DPL / 4; ++j) {
     const int c = 4 * sub + 32 * j;
     if (c < cols) {
-      const f32x4 v = {r.x[4 * j] * scale, r.x[4 * j + 1] * scale, r.x[4 * j + 2] * scale, r.x[4 * j + 3] * scale};
-      *reinterpret_cast<f32x4*>(p + c) = v;
+      quad v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = from_float<T>(r.x[4 * j + e] * scale);
+      *reinterpret_cast<quad*>(p + c) = v;
     }
   }
 }
@@ -83,8 +99,8 @@ __device__ __forceinline__ Vis make_vis(const MaskArgs& mk, const SeqInfo& si) {
 }
 
 // ---------------------------------------------------------------------------
-template <int DPL>
-__global__ void f32_fwd_kernel(const FwdArgs a) {
+template <typename T, int DPL>
+__global__ void valu_fwd_kernel(const FwdArgs a) {
   const int tid = threadIdx.x, sub = tid & 7;
   const int h = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
@@ -104,16 +120,16 @@ __global__ void f32_fwd_kernel(const FwdArgs a) {
   const bool dropout = a.drop.p > 0.f;
   DropoutState ds{};
   if (dropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
-  const float* qp = reinterpret_cast<const float*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
+  const T* qp = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
                     (int64_t)(si.q_start + mc) * a.sq.s;
-  const float* kb = reinterpret_cast<const float*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
+  const T* kb = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
                     (int64_t)si.k_start * a.sk.s;
-  const float* vb = reinterpret_cast<const float*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
+  const T* vb = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                     (int64_t)si.k_start * a.sv.s;
-  const float* bp = a.bias ? reinterpret_cast<const float*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
+  const T* bp = a.bias ? reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
                                  (int64_t)h * a.sb_h + (int64_t)mc * a.sb_m
                            : nullptr;
-  const Row<DPL> q = load_row<DPL>(qp, sub, a.head_dim, true);
+  const Row<DPL> q = load_row<DPL, T>(qp, sub, a.head_dim, true);
   Row<DPL> o;
 #pragma unroll
   for (int e = 0; e < DPL; ++e) o.x[e] = 0.f;
@@ -128,9 +144,9 @@ __global__ void f32_fwd_kernel(const FwdArgs a) {
     n_hi = m_last + vis.right < n_hi ? m_last + vis.right : n_hi;
   }
   for (int n = n_lo; n <= n_hi; ++n) {
-    const Row<DPL> kr = load_row<DPL>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true);
+    const Row<DPL> kr = load_row<DPL, T>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true);
     float s = dot8<DPL>(q, kr) * qk_scale;                                   // fwd_kernel_inner.py:166
-    if (bp) s += bp[(int64_t)n * a.sb_n] * kLog2e;                           // :187
+    if (bp) s += (float)bp[(int64_t)n * a.sb_n] * kLog2e;                           // :187
     if (!vis(m, n) || s == -__builtin_inff()) continue;                      // lanes of a row agree
     const float m_new = fmaxf(mi, s);
     const float alpha = fast_exp2(mi - m_new);                               // exp2(-inf) = 0 on the first key
@@ -139,7 +155,7 @@ __global__ void f32_fwd_kernel(const FwdArgs a) {
     mi = m_new;
     const bool keep = !dropout || dropout_keep1(ds, m, n);
     const float pv = keep ? p : 0.f;
-    const Row<DPL> vr = load_row<DPL>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true);
+    const Row<DPL> vr = load_row<DPL, T>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true);
 #pragma unroll
     for (int e = 0; e < DPL; ++e) o.x[e] = __builtin_fmaf(pv, vr.x[e], o.x[e] * alpha);
   }
@@ -147,16 +163,16 @@ __global__ void f32_fwd_kernel(const FwdArgs a) {
   const bool alive = li > 0.f;
   float inv = alive ? 1.0f / li : 0.f;
   if (dropout) inv *= ds.scale;                                              // fwd_kernel.py:573-580
-  float* op = reinterpret_cast<float*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
+  T* op = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
               (int64_t)(si.q_start + m) * a.so.s;
-  store_row<DPL>(op, o, sub, a.head_dim_v, inv);
+  store_row<DPL, T>(op, o, sub, a.head_dim_v, inv);
   if (a.lse && sub == 0)
     a.lse[lse_offset(si, h, a.hq) + m] = alive ? (mi + fast_log2(li)) * kLn2 : __builtin_inff();   // :610-612, :327-355
 }
 
 // ---------------------------------------------------------------------------
-template <int DPL>
-__global__ void f32_delta_kernel(const BwdArgs a) {
+template <typename T, int DPL>
+__global__ void valu_delta_kernel(const BwdArgs a) {
   const int tid = threadIdx.x, sub = tid & 7;
   const int h = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
@@ -164,17 +180,17 @@ __global__ void f32_delta_kernel(const BwdArgs a) {
   if (blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
   const bool row_ok = m < si.seqlen_q;
   const int mc = row_ok ? m : si.seqlen_q - 1;
-  const float* op = reinterpret_cast<const float*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
+  const T* op = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
                     (int64_t)(si.q_start + mc) * a.so.s;
-  const float* dop = reinterpret_cast<const float*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
+  const T* dop = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
                      (int64_t)h * a.sdo.h + (int64_t)(si.q_start + mc) * a.sdo.s;
-  const float d = dot8<DPL>(load_row<DPL>(op, sub, a.head_dim_v, true), load_row<DPL>(dop, sub, a.head_dim_v, true));
+  const float d = dot8<DPL>(load_row<DPL, T>(op, sub, a.head_dim_v, true), load_row<DPL, T>(dop, sub, a.head_dim_v, true));
   if (row_ok && sub == 0) a.delta[lse_offset(si, h, a.hq) + m] = d;
 }
 
 // One row of Q per lane group, all keys: dQ and dB.
-template <int DPL>
-__global__ void f32_dq_kernel(const BwdArgs a) {
+template <typename T, int DPL>
+__global__ void valu_dq_kernel(const BwdArgs a) {
   const int tid = threadIdx.x, sub = tid & 7;
   const int h = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
@@ -188,20 +204,20 @@ __global__ void f32_dq_kernel(const BwdArgs a) {
   DropoutState ds{};
   if (dropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
   const int64_t qoff = (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h + (int64_t)(si.q_start + mc) * a.sq.s;
-  const float* dop = reinterpret_cast<const float*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
+  const T* dop = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
                      (int64_t)h * a.sdo.h + (int64_t)(si.q_start + mc) * a.sdo.s;
-  const float* kb = reinterpret_cast<const float*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
+  const T* kb = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
                     (int64_t)si.k_start * a.sk.s;
-  const float* vb = reinterpret_cast<const float*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
+  const T* vb = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                     (int64_t)si.k_start * a.sv.s;
-  const float* bp = a.bias ? reinterpret_cast<const float*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
+  const T* bp = a.bias ? reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
                                  (int64_t)h * a.sb_h + (int64_t)mc * a.sb_m
                            : nullptr;
-  float* dbp = a.db ? reinterpret_cast<float*>(a.db) + (int64_t)si.batch_index * a.sdb_z + (int64_t)h * a.sdb_h +
+  T* dbp = a.db ? reinterpret_cast<T*>(a.db) + (int64_t)si.batch_index * a.sdb_z + (int64_t)h * a.sdb_h +
                           (int64_t)mc * a.sdb_m
                     : nullptr;
-  const Row<DPL> q = load_row<DPL>(reinterpret_cast<const float*>(a.q) + qoff, sub, a.head_dim, true);
-  const Row<DPL> dout = load_row<DPL>(dop, sub, a.head_dim_v, true);
+  const Row<DPL> q = load_row<DPL, T>(reinterpret_cast<const T*>(a.q) + qoff, sub, a.head_dim, true);
+  const Row<DPL> dout = load_row<DPL, T>(dop, sub, a.head_dim_v, true);
   const int64_t lo = lse_offset(si, h, a.hq) + mc;
   const float L = a.lse[lo] * kRcpLn2;                                       // bwd_kernel_dq.py:305
   const float delta = a.delta[lo];
@@ -212,10 +228,10 @@ __global__ void f32_dq_kernel(const BwdArgs a) {
   for (int n = 0; n < si.seqlen_k; ++n) {
     float dsv = 0.f;
     if (vis(m, n)) {
-      const Row<DPL> kr = load_row<DPL>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true);
-      const Row<DPL> vr = load_row<DPL>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true);
+      const Row<DPL> kr = load_row<DPL, T>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true);
+      const Row<DPL> vr = load_row<DPL, T>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true);
       float x = dot8<DPL>(q, kr) * qk_scale;
-      if (bp) x += bp[(int64_t)n * a.sb_n] * kLog2e;
+      if (bp) x += (float)bp[(int64_t)n * a.sb_n] * kLog2e;
       const float p = fast_exp2(x - L);                                      // bwd_inner_dq.py:158-160
       float dp = dot8<DPL>(dout, vr);
       if (dropout) dp = dropout_keep1(ds, m, n) ? dp * ds.scale : 0.f;      // :176-185
@@ -223,17 +239,17 @@ __global__ void f32_dq_kernel(const BwdArgs a) {
 #pragma unroll
       for (int e = 0; e < DPL; ++e) dq.x[e] = __builtin_fmaf(dsv, kr.x[e], dq.x[e]);
     }
-    if (dbp && row_ok && sub == 0) dbp[(int64_t)n * a.sdb_n] = dsv;          // :200-204; unvisited entries are zero
+    if (dbp && row_ok && sub == 0) dbp[(int64_t)n * a.sdb_n] = from_float<T>(dsv);          // :200-204; unvisited entries are zero
   }
   if (!row_ok) return;
-  float* dqp = reinterpret_cast<float*>(a.dq) + (int64_t)si.batch_index * a.sdq.z + (int64_t)h * a.sdq.h +
+  T* dqp = reinterpret_cast<T*>(a.dq) + (int64_t)si.batch_index * a.sdq.z + (int64_t)h * a.sdq.h +
                (int64_t)(si.q_start + m) * a.sdq.s;
-  store_row<DPL>(dqp, dq, sub, a.head_dim, a.sm_scale);                      // bwd_kernel_dq.py:374-376
+  store_row<DPL, T>(dqp, dq, sub, a.head_dim, a.sm_scale);                      // bwd_kernel_dq.py:374-376
 }
 
 // One row of K per lane group, all q-heads of its group and all queries: dK and dV.
-template <int DPL>
-__global__ void f32_dkdv_kernel(const BwdArgs a) {
+template <typename T, int DPL>
+__global__ void valu_dkdv_kernel(const BwdArgs a) {
   const int tid = threadIdx.x, sub = tid & 7;
   const int hk = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
@@ -244,10 +260,10 @@ __global__ void f32_dkdv_kernel(const BwdArgs a) {
   const Vis vis = make_vis(a.mask, si);
   const bool dropout = a.drop.p > 0.f;
   const int group = a.hq / a.hk;
-  const Row<DPL> kr = load_row<DPL>(reinterpret_cast<const float*>(a.k) + (int64_t)si.batch_index * a.sk.z +
+  const Row<DPL> kr = load_row<DPL, T>(reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
                                         (int64_t)hk * a.sk.h + (int64_t)(si.k_start + nc) * a.sk.s,
                                     sub, a.head_dim, true);
-  const Row<DPL> vr = load_row<DPL>(reinterpret_cast<const float*>(a.v) + (int64_t)si.batch_index * a.sv.z +
+  const Row<DPL> vr = load_row<DPL, T>(reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z +
                                         (int64_t)hk * a.sv.h + (int64_t)(si.k_start + nc) * a.sv.s,
                                     sub, a.head_dim_v, true);
   const float qk_scale = a.sm_scale * kLog2e;
@@ -258,20 +274,20 @@ __global__ void f32_dkdv_kernel(const BwdArgs a) {
     const int h = hk * group + g;
     DropoutState ds{};
     if (dropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
-    const float* qb = reinterpret_cast<const float*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
+    const T* qb = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
                       (int64_t)si.q_start * a.sq.s;
-    const float* dob = reinterpret_cast<const float*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
+    const T* dob = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
                        (int64_t)h * a.sdo.h + (int64_t)si.q_start * a.sdo.s;
-    const float* bb = a.bias ? reinterpret_cast<const float*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
+    const T* bb = a.bias ? reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
                                    (int64_t)h * a.sb_h + (int64_t)nc * a.sb_n
                              : nullptr;
     const int64_t lo = lse_offset(si, h, a.hq);
     for (int m = 0; m < si.seqlen_q; ++m) {
       if (!vis(m, n)) continue;                                              // lanes of a row agree
-      const Row<DPL> qr = load_row<DPL>(qb + (int64_t)m * a.sq.s, sub, a.head_dim, true);
-      const Row<DPL> dor = load_row<DPL>(dob + (int64_t)m * a.sdo.s, sub, a.head_dim_v, true);
+      const Row<DPL> qr = load_row<DPL, T>(qb + (int64_t)m * a.sq.s, sub, a.head_dim, true);
+      const Row<DPL> dor = load_row<DPL, T>(dob + (int64_t)m * a.sdo.s, sub, a.head_dim_v, true);
       float x = dot8<DPL>(qr, kr) * qk_scale;
-      if (bb) x += bb[(int64_t)m * a.sb_m] * kLog2e;
+      if (bb) x += (float)bb[(int64_t)m * a.sb_m] * kLog2e;
       const float p = fast_exp2(x - a.lse[lo + m] * kRcpLn2);               // bwd_inner_dk_dv.py:185-188
       const bool keep = !dropout || dropout_keep1(ds, m, n);
       const float pd = dropout ? (keep ? p * ds.scale : 0.f) : p;            // :194-201
@@ -286,12 +302,12 @@ __global__ void f32_dkdv_kernel(const BwdArgs a) {
     }
   }
   if (!row_ok) return;
-  float* dkp = reinterpret_cast<float*>(a.dk) + (int64_t)si.batch_index * a.sdk.z + (int64_t)hk * a.sdk.h +
+  T* dkp = reinterpret_cast<T*>(a.dk) + (int64_t)si.batch_index * a.sdk.z + (int64_t)hk * a.sdk.h +
                (int64_t)(si.k_start + n) * a.sdk.s;
-  float* dvp = reinterpret_cast<float*>(a.dv) + (int64_t)si.batch_index * a.sdv.z + (int64_t)hk * a.sdv.h +
+  T* dvp = reinterpret_cast<T*>(a.dv) + (int64_t)si.batch_index * a.sdv.z + (int64_t)hk * a.sdv.h +
                (int64_t)(si.k_start + n) * a.sdv.s;
-  store_row<DPL>(dkp, dk, sub, a.head_dim, a.sm_scale);                      // bwd_kernel_dk_dv.py:387-389
-  store_row<DPL>(dvp, dv, sub, a.head_dim_v, 1.0f);
+  store_row<DPL, T>(dkp, dk, sub, a.head_dim, a.sm_scale);                      // bwd_kernel_dk_dv.py:387-389
+  store_row<DPL, T>(dvp, dv, sub, a.head_dim_v, 1.0f);
 }
 
 int nseq_of(const SeqArgs& s, int batch) {
@@ -300,37 +316,53 @@ int nseq_of(const SeqArgs& s, int batch) {
 
 }  // namespace
 
-// head_dim: the compiled head dim (64, 128 or 256) that holds the tensors' head dims
-hipError_t run_fwd_f32(int head_dim, const FwdArgs& a, hipStream_t s) {
+// head_dim: 64, 128, 256 or 512, the one that holds the tensors' head dims.  The 16-bit types
+// are built for 512 only (the MFMA kernels serve the others).
+hipError_t run_fwd_valu(int dtype, int head_dim, const FwdArgs& a, hipStream_t s) {
   const dim3 grid((a.seq.max_seqlen_q + kRowsPerBlock - 1) / kRowsPerBlock, a.hq, nseq_of(a.seq, a.batch));
-  switch (head_dim) {
-    case 64: hipLaunchKernelGGL(f32_fwd_kernel<8>, grid, dim3(256), 0, s, a); break;
-    case 128: hipLaunchKernelGGL(f32_fwd_kernel<16>, grid, dim3(256), 0, s, a); break;
-    case 256: hipLaunchKernelGGL(f32_fwd_kernel<32>, grid, dim3(256), 0, s, a); break;
-    default: return hipErrorNotSupported;
+  if (dtype == kDtypeF32) {
+    switch (head_dim) {
+      case 64: hipLaunchKernelGGL((valu_fwd_kernel<float, 8>), grid, dim3(256), 0, s, a); break;
+      case 128: hipLaunchKernelGGL((valu_fwd_kernel<float, 16>), grid, dim3(256), 0, s, a); break;
+      case 256: hipLaunchKernelGGL((valu_fwd_kernel<float, 32>), grid, dim3(256), 0, s, a); break;
+      case 512: hipLaunchKernelGGL((valu_fwd_kernel<float, 64>), grid, dim3(256), 0, s, a); break;
+      default: return hipErrorNotSupported;
+    }
+  } else if (head_dim == 512) {
+    if (dtype == kDtypeBF16) hipLaunchKernelGGL((valu_fwd_kernel<bf16_t, 64>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((valu_fwd_kernel<f16_t, 64>), grid, dim3(256), 0, s, a);
+  } else {
+    return hipErrorNotSupported;
   }
   return hipGetLastError();
 }
 
 // kernel_slot: 0 delta, 1 dK/dV, 2 dQ (and dB)
-hipError_t run_bwd_f32(int head_dim, int kernel_slot, const BwdArgs& a, hipStream_t s) {
+hipError_t run_bwd_valu(int dtype, int head_dim, int kernel_slot, const BwdArgs& a, hipStream_t s) {
   const int nseq = nseq_of(a.seq, a.batch);
   const dim3 gq((a.seq.max_seqlen_q + kRowsPerBlock - 1) / kRowsPerBlock, a.hq, nseq);
   const dim3 gk((a.seq.max_seqlen_k + kRowsPerBlock - 1) / kRowsPerBlock, a.hk, nseq);
-#define FA_F32_LAUNCH(DPL)                                                                      \
-  switch (kernel_slot) {                                                                        \
-    case 0: hipLaunchKernelGGL(f32_delta_kernel<DPL>, gq, dim3(256), 0, s, a); break;           \
-    case 1: hipLaunchKernelGGL(f32_dkdv_kernel<DPL>, gk, dim3(256), 0, s, a); break;            \
-    case 2: hipLaunchKernelGGL(f32_dq_kernel<DPL>, gq, dim3(256), 0, s, a); break;              \
-    default: return hipErrorInvalidValue;                                                       \
+#define FA_VALU_LAUNCH(T, DPL)                                                                     \
+  switch (kernel_slot) {                                                                           \
+    case 0: hipLaunchKernelGGL((valu_delta_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;        \
+    case 1: hipLaunchKernelGGL((valu_dkdv_kernel<T, DPL>), gk, dim3(256), 0, s, a); break;         \
+    case 2: hipLaunchKernelGGL((valu_dq_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;           \
+    default: return hipErrorInvalidValue;                                                          \
   }
-  switch (head_dim) {
-    case 64: FA_F32_LAUNCH(8) break;
-    case 128: FA_F32_LAUNCH(16) break;
-    case 256: FA_F32_LAUNCH(32) break;
-    default: return hipErrorNotSupported;
+  if (dtype == kDtypeF32) {
+    switch (head_dim) {
+      case 64: FA_VALU_LAUNCH(float, 8) break;
+      case 128: FA_VALU_LAUNCH(float, 16) break;
+      case 256: FA_VALU_LAUNCH(float, 32) break;
+      case 512: FA_VALU_LAUNCH(float, 64) break;
+      default: return hipErrorNotSupported;
+    }
+  } else if (head_dim == 512) {
+    if (dtype == kDtypeBF16) { FA_VALU_LAUNCH(bf16_t, 64) } else { FA_VALU_LAUNCH(f16_t, 64) }
+  } else {
+    return hipErrorNotSupported;
   }
-#undef FA_F32_LAUNCH
+#undef FA_VALU_LAUNCH
   return hipGetLastError();
 }
 

@@ -44,7 +44,7 @@ def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.
                                  scale=None, enable_gqa=False, extra=None):
     """Same signature and semantics as torch.nn.functional.scaled_dot_product_attention for
     4-D fp16/bf16 CUDA tensors (B, H, L, E), with these limits: the head dims (of q/k, and of
-    v) are multiples of 8 up to 256; a boolean mask is turned into an additive one
+    v) are multiples of 8 up to 512 (fp32 and head dims above 256 take slow kernels); a boolean mask is turned into an additive one
     (0 / -inf), and a query row that the mask hides completely yields zeros instead of NaN;
     dropout uses the operators' Philox stream (seed/offsets in `extra`), not torch's generator.
     """

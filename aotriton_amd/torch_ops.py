@@ -133,7 +133,7 @@ flash_attention_forward.register_autograd(_backward, setup_context=_setup_contex
 def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False,
                                  scale=None, enable_gqa=False):
     """torch.nn.functional.scaled_dot_product_attention on the custom ops above: 4-D fp16/bf16
-    CUDA tensors (B, H, L, E), head dims multiples of 8 up to 256.  A boolean mask becomes an
+    CUDA tensors (B, H, L, E), head dims multiples of 8 up to 512.  A boolean mask becomes an
     additive one (0 / -inf); a query row that the mask hides completely yields zeros instead
     of NaN; dropout draws seed and offset from torch's CUDA generator (so torch.manual_seed
     governs it) but uses the operators' Philox stream, not the one of torch's own kernels.

@@ -55,7 +55,7 @@ enum fa_error {
   FA_ERROR_INVALID_SYMBOL = 13,           /* params_version mismatch                     */
   FA_ERROR_NO_BINARY_FOR_GPU = 209,       /* device is not gfx950                        */
   FA_ERROR_PEER_ACCESS_UNSUPPORTED = 217, /* a forced backend cannot take this input     */
-  FA_ERROR_NOT_SUPPORTED = 801,           /* functional not built (head dim, stride, ..) */
+  FA_ERROR_NOT_SUPPORTED = 801,           /* functional not built (head dim > 512, stride, ..) */
 };
 
 /* TensorView<4|2|1|0>, include/aotriton/util.h:77-210. */

@@ -142,6 +142,18 @@ def test_fp32_inputs(case):
               bias=c['bias'], bshd=c['bshd'], Dv=c['Dv'], bwd_backend=0)
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('D,Dv', [(512, None), (320, 264), (128, 512)])
+def test_head_dims_up_to_512(dtype, D, Dv):
+    # above 256 every type runs on the vector-ALU kernels (the reference compiles head dim 512,
+    # modules/flash/aot/_common.py:10-14)
+    _run_case(1, 4, 2, 150, 131, D, dtype, (40, 0), Dv=Dv, bwd_backend=0)
+
+
+def test_head_dim_512_with_bias_and_dropout():
+    _run_case(1, 2, 2, 100, 100, 512, torch.bfloat16, True, dropout_p=0.2, bias=True, bwd_backend=0)
+
+
 def test_fp32_has_no_fused_backend():
     from aotriton_amd.autograd import attention, AttentionExtraArgs
     q, k, v, _, do = make_inputs(1, 2, 2, 64, 64, 64, torch.float32, DEV)
