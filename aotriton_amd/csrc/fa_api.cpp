@@ -376,10 +376,17 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
   const int mt = (s.max_sq + t.block_m - 1) / t.block_m, nt = (s.max_sk + t.block_n - 1) / t.block_n;
-  // 1-D grids of the main kernels: 8 XCDs x (heads per XCD, rounded up to whole groups) x items per head
+  // 1-D work lists of the main kernels: 8 XCDs x (heads per XCD, rounded up to whole groups) x
+  // items per head.  The fused kernel launches one workgroup per item, and so do dK/dV and dQ
+  // with a bias or at D = 256; otherwise they run persistent workgroups, one per CU (256 CUs assumed
+  // here) and at most one per item.
   auto grid1d = [&](int heads, int zg, int items) {
     const int per_xcd = (nz * heads + fa::kNumXcd - 1) / fa::kNumXcd;
     return fa::kNumXcd * ((per_xcd + zg - 1) / zg) * zg * items;
+  };
+  auto persistent = [&](int items_total) {
+    const int per_xcd = items_total / fa::kNumXcd;
+    return s.bias || s.d >= 256 ? items_total : fa::kNumXcd * (per_xcd < 32 ? per_xcd : 32);
   };
   const int ratio = s.hq / s.hk;
   out->grid[1] = 1;
@@ -390,8 +397,8 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
     out->grid[2] = nz;
   } else switch (kernel_slot) {
     case 0: out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz; break;
-    case 1: out->grid[0] = grid1d(s.hk, 2, nt); break;
-    case 2: out->grid[0] = grid1d(s.hq, ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2, mt); break;
+    case 1: out->grid[0] = persistent(grid1d(s.hk, 2, nt)); break;
+    case 2: out->grid[0] = persistent(grid1d(s.hq, ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2, mt)); break;
     default: out->grid[0] = grid1d(s.hk, 2, nt + mt * ratio); break;
   }
   out->backend_index = be;
@@ -502,6 +509,7 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
   a.drop = dropout_args(p->dropout_p, p->philox_seed_ptr, p->philox_offset1, p->philox_offset2);
+  a.num_cu = dev->num_cu;
 
   const int dt = p->Q.dtype;
   FA_LOG(4, "attn_bwd: backend=%d slot=%d D=%d windowed=%d bias=%d dropout=%d nseq=%d", backend,

@@ -75,6 +75,8 @@ struct BwdArgs {
   int32_t num_zh;        // (batch or sequences) x heads of the launched kernel's grid
   int32_t zh_per_xcd;    // ceil(num_zh / 8)
   int32_t zh_group;      // heads walked together on one XCD
+  int32_t num_cu;        // CUs of the device (host fills it in)
+  int32_t items_per_xcd; // work items (incl. padding of the last group) per XCD
 };
 
 struct EncodedSoftmaxArgs {

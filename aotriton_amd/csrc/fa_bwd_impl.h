@@ -1031,35 +1031,51 @@ template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kD
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dkdv_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  // 1-D grid: each XCD owns a contiguous range of (batch, kv-head) pairs and walks
-  // them in pairs, K tiles in ascending order (the heaviest causal tile first), so the
-  // Q/dO stream of the heads in flight stays in that XCD's L2.
-  const int xcd = blockIdx.x % kNumXcd, li = blockIdx.x / kNumXcd;
+  // Persistent workgroups, one per CU (a relaunch per item costs a dispatch gap of several
+  // microseconds on every CU).  Each XCD owns a contiguous range of (batch, kv-head)
+  // pairs and walks them in pairs, K tiles in ascending order (the heaviest causal tile
+  // first), so the Q/dO stream of the heads in flight stays in that XCD's L2; the
+  // workgroups of the XCD take the items in serpentine order (worker p takes p,
+  // 2P-1-p, 2P+p, ...), which pairs heavy with light items.
+  const int xcd = blockIdx.x % kNumXcd, p = blockIdx.x / kNumXcd, workers = gridDim.x / kNumXcd;
   const int per_group = a.zh_group * a.num_n_tiles;
-  const int gi = li / per_group, gr = li % per_group;
-  const int zl = gi * a.zh_group + gr % a.zh_group;
-  const int zh = xcd * a.zh_per_xcd + zl;
-  if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
-  int z, hk;
-  split_zh(zh, a.num_zh / a.hk, 1, z, hk);
-  dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad>(a, hk, gr / a.zh_group, z, smem_raw);
+  // (D = 256 is launched with one workgroup per item: the loop would cost registers there)
+  for (int r = 0; D >= 256 ? r < 1 : r * workers < a.items_per_xcd; ++r) {
+    const int li = r * workers + ((r & 1) ? workers - 1 - p : p);
+    if (li >= a.items_per_xcd) continue;
+    const int gi = li / per_group, gr = li % per_group;
+    const int zl = gi * a.zh_group + gr % a.zh_group;
+    const int zh = xcd * a.zh_per_xcd + zl;
+    if (zl >= a.zh_per_xcd || zh >= a.num_zh) continue;
+    int z, hk;
+    split_zh(zh, a.num_zh / a.hk, 1, z, hk);
+    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad>(a, hk, gr / a.zh_group, z, smem_raw);
+    __syncthreads();     // the next item reuses the LDS stages
+  }
 }
 
 template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dq_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-  // same walk as the forward kernel: (batch, q-head) pairs per XCD, heaviest Q tile first
-  const int xcd = blockIdx.x % kNumXcd, li = blockIdx.x / kNumXcd;
+  // persistent workgroups with the same walk as the forward kernel: (batch, q-head) pairs
+  // per XCD, heaviest Q tile first, serpentine over the workgroups of the XCD
+  const int xcd = blockIdx.x % kNumXcd, p = blockIdx.x / kNumXcd, workers = gridDim.x / kNumXcd;
   const int per_group = a.zh_group * a.num_m_tiles;
-  const int gi = li / per_group, gr = li % per_group;
-  const int zl = gi * a.zh_group + gr % a.zh_group;
-  const int zh = xcd * a.zh_per_xcd + zl;
-  if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
-  const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
-  int z, h;
-  split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
-  dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false, kPad>(a, h, mt, z, smem_raw);
+  // (D = 256 is launched with one workgroup per item: the loop would cost registers there)
+  for (int r = 0; D >= 256 ? r < 1 : r * workers < a.items_per_xcd; ++r) {
+    const int li = r * workers + ((r & 1) ? workers - 1 - p : p);
+    if (li >= a.items_per_xcd) continue;
+    const int gi = li / per_group, gr = li % per_group;
+    const int zl = gi * a.zh_group + gr % a.zh_group;
+    const int zh = xcd * a.zh_per_xcd + zl;
+    if (zl >= a.zh_per_xcd || zh >= a.num_zh) continue;
+    const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
+    int z, h;
+    split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
+    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false, kPad>(a, h, mt, z, smem_raw);
+    __syncthreads();     // the next item reuses the LDS stages
+  }
 }
 
 // Per (batch, kv-head): num_n_tiles dK/dV items followed by num_m_tiles*(Hq/Hk) dQ items
@@ -1097,6 +1113,20 @@ void bwd_fused_kernel(const BwdArgs a) {
 // ---------------------------------------------------------------------------
 inline int bwd_nseq(const BwdArgs& a) {
   return a.seq.num_seqlens != 0 ? (a.seq.num_seqlens < 0 ? -a.seq.num_seqlens : a.seq.num_seqlens) : a.batch;
+}
+
+// Workgroups per XCD of the dK/dV and dQ kernels: one per CU, at most one per item.  With a
+// bias the kernels get one workgroup per item instead (the loop of a workgroup then runs
+// once): measured at B2 H16 S8192 D256 with window, bias, dB and dropout the persistent
+// grid was 10 % slower, while it gains 1 % at the headline shape and 12 % on packed
+// sequences of very different lengths.  D = 256 also gets one workgroup per item: its
+// dK/dV kernel has no register to spare for the loop.
+template <int D>
+inline int persistent_workers(const BwdArgs& a) {
+  if (a.bias != nullptr || D >= 256) return a.items_per_xcd;
+  int w = (a.num_cu > 0 ? a.num_cu : 256) / kNumXcd;
+  if (w < 1) w = 1;
+  return w > a.items_per_xcd ? a.items_per_xcd : w;
 }
 
 template <typename K>
@@ -1138,7 +1168,8 @@ hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dro
   a.num_zh = bwd_nseq(a) * a.hk;
   a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
   a.zh_group = 2;
-  dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles));
+  a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles;
+  dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
 #define FA_CALL(W, B, P) launch_with_lds(bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>, grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
@@ -1152,7 +1183,8 @@ hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropo
   a.num_zh = bwd_nseq(a) * a.hq;
   a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
   a.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
-  dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_m_tiles));
+  a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_m_tiles;
+  dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
 #define FA_CALL(W, B, P) launch_with_lds(bwd_dq_kernel<T, D, NW, BN, W, B, P, kPad>, grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL

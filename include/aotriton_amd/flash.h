@@ -239,7 +239,8 @@ FA_API int fa_validate_fwd(const fa_fwd_params* params, int32_t params_version,
 FA_API int fa_validate_bwd(const fa_bwd_params* params, int32_t params_version,
                            const fa_options* options);
 
-/* Tile/grid the library would use (host only, num_cu = CU count to assume). */
+/* Tile/grid the library would use (host only, num_cu = CU count to assume; the backward
+ * query assumes 256 CUs). */
 FA_API int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu,
                                fa_kernel_config* out);
 FA_API int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options,
