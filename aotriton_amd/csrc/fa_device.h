@@ -27,6 +27,7 @@ using vec = T __attribute__((ext_vector_type(N)));
 
 using f32x16 = vec<float, 16>;
 using f32x4 = vec<float, 4>;
+using u32x4_t = vec<unsigned, 4>;   // payload type of the 16-byte buffer loads and stores
 
 constexpr float kLog2e = 1.44269504089f;       // modules/flash/kernel/fwd_kernel.py:422
 constexpr float kLn2 = 0.6931471824645996f;    // modules/flash/kernel/fwd_kernel.py:610-612

@@ -13,6 +13,9 @@
 // Both tiles are staged row-major.  K rows are padded by 16 B (conflict-free
 // 16-byte row reads); V rows are padded by 64 B so that the transposing LDS reads
 // (ds_read_b64_tr_b16: 4 rows x 64 B per half-wave) sweep all banks once.
+// Q rows on the way in and O rows on the way out pass through a private LDS area of
+// the wave (32 rows, +16 B per row): global memory sees whole rows in 16-byte pieces
+// of consecutive lanes, while the MFMA layouts want one row per lane.
 #pragma once
 #include <type_traits>
 
@@ -20,14 +23,16 @@
 
 namespace fa {
 
-template <int D, int BN>
+template <int D, int BN, int NW>
 struct FwdSmem {
   static constexpr int KSTR = D + 8;     // +16 B per row
   static constexpr int VSTR = D + 32;    // +64 B per row
   static constexpr int K_ELEMS = BN * KSTR;
   static constexpr int V_ELEMS = BN * VSTR;
   static constexpr int STAGES = 2;
-  static constexpr int BYTES = STAGES * (K_ELEMS + V_ELEMS) * 2;
+  static constexpr int ROWS_OFF = STAGES * (K_ELEMS + V_ELEMS) * 2;   // the waves' row areas
+  static constexpr int ROW_STR = D * 2 + 16;                          // bytes per staged Q / O row
+  static constexpr int BYTES = ROWS_OFF + NW * 32 * ROW_STR;
 };
 
 // One Q tile (BM rows of head h of sequence z) against all its visible K/V tiles.
@@ -36,7 +41,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   using Tr = Traits<T>;
   using op_t = typename Tr::op_t;
   using q4_t = typename Tr::q4_t;
-  using SM = FwdSmem<D, BN>;
+  using SM = FwdSmem<D, BN, NW>;
   constexpr int NT = NW * 64;
   constexpr int BM = NW * 32;
   constexpr int KS = D / 16;    // k-steps of S^T = K Q^T
@@ -91,14 +96,31 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   }
 
   // ---- Q rows as the B operand, resident for the whole tile ------------------
-  const T* qptr = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z +
-                  (int64_t)h * a.sq.h + (int64_t)(si.q_start + row_c) * a.sq.s;
+  // The wave's 32 rows come in as whole rows (16 bytes per lane, consecutive lanes along a
+  // row) through its LDS area; rows past the sequence and columns past the tensors' head
+  // dim read as zero (head dims are rounded up to D).
+  constexpr int LPRQ = D / 8;             // 16-byte pieces per row
+  constexpr int RPQ = 64 / LPRQ;          // rows per wave-wide access
+  char* rowbuf = smem_raw + SM::ROWS_OFF + wave * 32 * SM::ROW_STR;
+  const int wrows = si.seqlen_q - q0 - wave * 32 < 32 ? si.seqlen_q - q0 - wave * 32 : 32;   // may be <= 0
+  const int rq = lane / LPRQ, cq = lane % LPRQ;
   op_t qreg[KS];
+  {
+    const T* qw = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
+                  (int64_t)(si.q_start + q0 + wave * 32) * a.sq.s;
+    const auto qrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qw), 0,
+                                                       wrows > 0 ? ((wrows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
+    const int qvoff = cq * 8 < d_qk ? rq * (int)a.sq.s * 2 + cq * 16 : kVoffOutOfRange;
+    op_t qin[32 / RPQ];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    // columns past the tensors' head dim are zero (head dims are rounded up to D)
-    const op_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    qreg[ks] = 16 * ks + 8 * hi < d_qk ? *reinterpret_cast<const op_t*>(qptr + 16 * ks + 8 * hi) : zero8;
+    for (int i = 0; i < 32 / RPQ; ++i)
+      qin[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(qrs, qvoff, i * RPQ * (int)a.sq.s * 2, 0));
+#pragma unroll
+    for (int i = 0; i < 32 / RPQ; ++i)
+      *reinterpret_cast<op_t*>(rowbuf + (i * RPQ + rq) * SM::ROW_STR + cq * 16) = qin[i];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qreg[ks] = *reinterpret_cast<const op_t*>(rowbuf + c * SM::ROW_STR + (16 * ks + 8 * hi) * 2);
   }
 
   const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
@@ -409,19 +431,30 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   const bool alive = l > 0.f;
   float inv = alive ? 1.0f / l : 0.f;
   if (kDropout) inv *= ds.scale;          // fwd_kernel.py:573-575
-  if (row_ok) {
+  // O rows leave the way the Q rows came: through the wave's LDS area, as whole rows
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        q4_t t4;
+    for (int g = 0; g < 4; ++g) {
+      q4_t t4;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(o[db][4 * g + r] * inv);
-        if (32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
-      }
-    if (lse_ptr && hi == 0)
-      lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
+      for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(o[db][4 * g + r] * inv);
+      *reinterpret_cast<q4_t*>(rowbuf + c * SM::ROW_STR + (32 * db + 8 * g + 4 * hi) * 2) = t4;
+    }
+  {
+    T* ow = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
+            (int64_t)(si.q_start + q0 + wave * 32) * a.so.s;
+    const auto ors = __builtin_amdgcn_make_buffer_rsrc(ow, 0, wrows > 0 ? ((wrows - 1) * (int)a.so.s + d_v) * 2 : 0,
+                                                       0x00020000);
+    const int ovoff = cq * 8 < d_v ? rq * (int)a.so.s * 2 + cq * 16 : kVoffOutOfRange;
+#pragma unroll
+    for (int i = 0; i < 32 / RPQ; ++i) {
+      const op_t x = *reinterpret_cast<const op_t*>(rowbuf + (i * RPQ + rq) * SM::ROW_STR + cq * 16);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), ors, ovoff, i * RPQ * (int)a.so.s * 2, 0);
+    }
   }
+  if (row_ok && lse_ptr && hi == 0)
+    lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
 }
 
 // Persistent workgroups: the grid holds one workgroup per CU.  Consecutive workgroup
@@ -474,7 +507,7 @@ template <typename T, int D, bool kWindowed, bool kBias, bool kDropout, bool kPa
 hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
   constexpr int NW = FwdTile<D>::NW, BN = FwdTile<D>::BN;
   auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>;
-  constexpr int smem = FwdSmem<D, BN>::BYTES;
+  constexpr int smem = FwdSmem<D, BN, NW>::BYTES;
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);

@@ -6,7 +6,7 @@
 namespace fa {
 
 template <int D> static TileShape fwd_shape() {
-  return TileShape{FwdTile<D>::NW * 32, FwdTile<D>::BN, FwdTile<D>::NW, FwdSmem<D, FwdTile<D>::BN>::BYTES};
+  return TileShape{FwdTile<D>::NW * 32, FwdTile<D>::BN, FwdTile<D>::NW, FwdSmem<D, FwdTile<D>::BN, FwdTile<D>::NW>::BYTES};
 }
 
 TileShape fwd_tile_shape(int head_dim) {
