@@ -74,9 +74,10 @@ bool is_16bit(int dt) { return dt == FA_DTYPE_FLOAT16 || dt == FA_DTYPE_BFLOAT16
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// rank-4 activation tensor: non-null, unit last stride, 16-byte aligned rows
+// rank-4 activation tensor: non-null unless it has no element, unit last stride, 16-byte aligned rows
 int check_act(const fa_tensor4& t, int dtype) {
-  if (t.ptr == nullptr) return FA_ERROR_INVALID_VALUE;
+  const bool empty = (t.sizes[0] == 0 || t.sizes[1] == 0 || t.sizes[2] == 0) && t.sizes[3] > 0;
+  if (t.ptr == nullptr && !empty) return FA_ERROR_INVALID_VALUE;
   if (t.dtype != dtype) return FA_ERROR_INVALID_VALUE;
   if (t.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
   if (!aligned16(t.ptr)) return FA_ERROR_NOT_SUPPORTED;
@@ -232,7 +233,9 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
         p->DV.sizes[i] != p->V.sizes[i])
       return FA_ERROR_INVALID_VALUE;
   }
-  if (p->L.ptr == nullptr || p->L.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  // without a query row L and delta hold nothing and may be null
+  const bool no_query = p->Q.sizes[0] == 0 || p->Q.sizes[2] == 0;
+  if ((p->L.ptr == nullptr && !no_query) || p->L.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
   if (p->DB.ptr != nullptr) {
     if (!s.bias) return FA_ERROR_INVALID_VALUE;
     if (p->DB.dtype != dt) return FA_ERROR_INVALID_VALUE;
@@ -521,7 +524,8 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
     fa_tensor2 delta = p->D.eager;
     bool acquired = false;
     if (delta.ptr == nullptr) {
-      if (lazy->acquire(lazy, &delta) != 0 || delta.ptr == nullptr) return FA_ERROR_INVALID_VALUE;
+      const bool no_query = p->Q.sizes[0] == 0 || p->Q.sizes[2] == 0;
+      if (lazy->acquire(lazy, &delta) != 0 || (delta.ptr == nullptr && !no_query)) return FA_ERROR_INVALID_VALUE;
       acquired = true;
     }
     a.delta = static_cast<float*>(delta.ptr);

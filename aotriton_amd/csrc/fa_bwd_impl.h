@@ -1131,6 +1131,7 @@ inline int persistent_workers(const BwdArgs& a) {
 
 template <typename K>
 hipError_t launch_with_lds(K kern, dim3 grid, int nthreads, int smem, hipStream_t stream, const BwdArgs& a) {
+  if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;   // an empty tensor: nothing to write
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -1156,6 +1157,7 @@ template <typename T, int D>
 hipError_t launch_bwd_preprocess(const BwdArgs& a, hipStream_t stream) {
   constexpr int ROWS = 256 / (D / 8);
   dim3 grid((a.seq.max_seqlen_q + ROWS - 1) / ROWS, a.hq, bwd_nseq(a));
+  if (grid.x == 0 || grid.z == 0) return hipSuccess;
   hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), grid, dim3(256), 0, stream, a);
   return hipGetLastError();
 }

@@ -508,6 +508,7 @@ hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
   constexpr int NW = FwdTile<D>::NW, BN = FwdTile<D>::BN;
   auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>;
   constexpr int smem = FwdSmem<D, BN, NW>::BYTES;
+  if (grid.x == 0) return hipSuccess;      // no batch, no head or no query row: nothing to write
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);

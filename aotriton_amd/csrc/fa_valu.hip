@@ -320,6 +320,7 @@ int nseq_of(const SeqArgs& s, int batch) {
 // are built for 512 only (the MFMA kernels serve the others).
 hipError_t run_fwd_valu(int dtype, int head_dim, const FwdArgs& a, hipStream_t s) {
   const dim3 grid((a.seq.max_seqlen_q + kRowsPerBlock - 1) / kRowsPerBlock, a.hq, nseq_of(a.seq, a.batch));
+  if (grid.x == 0 || grid.z == 0) return hipSuccess;      // an empty tensor: nothing to write
   if (dtype == kDtypeF32) {
     switch (head_dim) {
       case 64: hipLaunchKernelGGL((valu_fwd_kernel<float, 8>), grid, dim3(256), 0, s, a); break;
@@ -342,6 +343,8 @@ hipError_t run_bwd_valu(int dtype, int head_dim, int kernel_slot, const BwdArgs&
   const int nseq = nseq_of(a.seq, a.batch);
   const dim3 gq((a.seq.max_seqlen_q + kRowsPerBlock - 1) / kRowsPerBlock, a.hq, nseq);
   const dim3 gk((a.seq.max_seqlen_k + kRowsPerBlock - 1) / kRowsPerBlock, a.hk, nseq);
+  const dim3& g = kernel_slot == 1 ? gk : gq;
+  if (g.x == 0 || g.z == 0) return hipSuccess;            // an empty tensor: nothing to write
 #define FA_VALU_LAUNCH(T, DPL)                                                                     \
   switch (kernel_slot) {                                                                           \
     case 0: hipLaunchKernelGGL((valu_delta_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;        \

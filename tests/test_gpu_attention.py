@@ -169,6 +169,32 @@ def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
     _run_case(2, 2, 2, 300, 140, 128, torch.bfloat16, causal)
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('backend', [0, 1])
+@pytest.mark.parametrize('shape', [(0, 16, 16), (2, 0, 16), (2, 16, 0)])
+def test_empty_tensors(shape, backend, dtype):
+    # no batch element, no query row, no key: the calls succeed; without a key O = 0,
+    # LSE = +inf and dQ = 0; without a query dK = dV = 0
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    if dtype == torch.float32 and backend == 1:
+        pytest.skip('fp32 has the split backend only')
+    B, Sq, Sk = shape
+    H, D = 2, 64
+    q = torch.randn(B, H, Sq, D, device=DEV).to(dtype).requires_grad_()
+    k = torch.randn(B, H, Sk, D, device=DEV).to(dtype).requires_grad_()
+    v = torch.randn(B, H, Sk, D, device=DEV).to(dtype).requires_grad_()
+    for causal in (False, True):
+        q.grad = k.grad = v.grad = None
+        ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend)
+        o, _, L = attention(q, k, v, None, causal, 0.125, 0.0, ext)
+        o.backward(torch.randn(B, H, Sq, D, device=DEV).to(dtype))
+        torch.cuda.synchronize()
+        assert o.shape == (B, H, Sq, D) and L.shape == (B * H, Sq)
+        assert torch.count_nonzero(o) == 0 and bool(torch.isposinf(L).all())
+        for g, t in ((q.grad, q), (k.grad, k), (v.grad, v)):
+            assert g.shape == t.shape and torch.count_nonzero(g) == 0 and not bool(torch.isnan(g).any())
+
+
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('causal', [False, True])
 def test_row_maximum_grows_along_keys(dtype, causal):

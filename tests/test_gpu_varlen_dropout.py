@@ -55,6 +55,62 @@ def test_compact_varlen_gqa(dtype, D, causal, backend):
     check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_compact_varlen_with_empty_sequences(dtype, causal, backend):
+    # sequences without queries, without keys and without both among ordinary ones, and
+    # query and key lengths that differ: rows without a key give O = 0, LSE = +inf, dQ = 0;
+    # keys without a query give dK = dV = 0
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
+    from oracle import fa_ref
+    if dtype == torch.float32 and backend == 1:
+        pytest.skip('fp32 has the split backend only')
+    lq = np.array([5, 0, 70, 0, 33, 130])
+    lk = np.array([9, 64, 0, 0, 33, 40])
+    Hq, Hk, D = 4, 2, 64
+    cq = [0] + np.cumsum(lq).tolist()
+    ck = [0] + np.cumsum(lk).tolist()
+    g = torch.Generator().manual_seed(11)
+    mk = lambda H, T: torch.randn(1, T, H, D, generator=g).to(dtype).to(DEV).transpose(1, 2)
+    q, do = mk(Hq, cq[-1]), mk(Hq, cq[-1])
+    k, v = mk(Hk, ck[-1]), mk(Hk, ck[-1])
+    sm = 1.0 / math.sqrt(D)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend)
+    o, _, L = attention_varlen(qg, kg, vg, lq, lk, causal, sm, 0.0, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    ct, wl, wr = flash.translate_causal(causal)
+    hp = torch.float64 if dtype == torch.float32 else torch.float32
+    f = lambda t: t.to(hp)
+    for i in range(len(lq)):
+        sq, sk = slice(cq[i], cq[i + 1]), slice(ck[i], ck[i + 1])
+        if lq[i] == 0:
+            assert torch.count_nonzero(kg.grad[:, :, sk]) == 0 and torch.count_nonzero(vg.grad[:, :, sk]) == 0
+            continue
+        if lk[i] == 0:
+            assert torch.count_nonzero(o[:, :, sq]) == 0 and bool(torch.isposinf(L[:, sq]).all())
+            assert torch.count_nonzero(qg.grad[:, :, sq]) == 0
+            continue
+        ro, rl, _ = fa_ref.attn_fwd_ref(f(q[:, :, sq]), f(k[:, :, sk]), f(v[:, :, sk]), None, sm, ct, wl, wr)
+        lo, ll, _ = fa_ref.attn_fwd_ref(q[:, :, sq], k[:, :, sk], v[:, :, sk], None, sm, ct, wl, wr)
+        check(f'out[{i}]', o[:, :, sq], ro, lo, FUDGE['out'])
+        live = torch.isfinite(rl[0])
+        assert torch.equal(torch.isinf(L[:, sq]), ~live)
+        assert (L[:, sq][live] - rl[0][live]).abs().max().item() <= LSE_ATOL
+        rg = fa_ref.attn_bwd_ref(f(q[:, :, sq]), f(k[:, :, sk]), f(v[:, :, sk]), None, sm, ro, f(do[:, :, sq]), rl,
+                                 ct, wl, wr)
+        lg = fa_ref.attn_bwd_ref(q[:, :, sq], k[:, :, sk], v[:, :, sk], None, sm, lo, do[:, :, sq],
+                                 ll.to(dtype), ct, wl, wr)
+        check(f'dq[{i}]', qg.grad[:, :, sq], rg[0], lg[0], FUDGE['dq'])
+        check(f'dk[{i}]', kg.grad[:, :, sk], rg[1], lg[1], FUDGE['dk'])
+        check(f'dv[{i}]', vg.grad[:, :, sk], rg[2], lg[2], FUDGE['dv'])
+    assert not bool(torch.isnan(o).any()) and not bool(torch.isnan(qg.grad).any())
+    assert not bool(torch.isnan(kg.grad).any()) and not bool(torch.isnan(vg.grad).any())
+
+
 def test_compact_varlen_fp32():
     # packed sequences through the fp32 kernels; oracle in fp64 against fp32
     from aotriton_amd import flash
