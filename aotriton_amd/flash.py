@@ -58,8 +58,18 @@ def translate_causal(causal, v3_api=True):
     return causal_type, window_left, window_right
 
 
+_DTYPES = {}
+
+
 def cast_dtype(dtype):
     """aotriton_flash.py:83-91."""
+    r = _DTYPES.get(dtype)
+    if r is None:
+        r = _DTYPES[dtype] = _cast_dtype(dtype)
+    return r
+
+
+def _cast_dtype(dtype):
     assert not dtype.is_complex
     bits = dtype.itemsize * 8
     if dtype.is_floating_point:
@@ -103,7 +113,7 @@ def _fill_fwd(params, q, k, v, b, sm_scale, M, o, dropout_p, philox_seed, philox
     params.V = mk_aotensor(v)
     params.B = mk_aotensor(b if (b is not None and b.numel() > 0) else None, if_empty_then_like=q)
     params.Sm_scale = float(sm_scale)
-    params.L = mk_aotensor(M, if_empty_then_like=q.new_empty((0, 0)))
+    params.L = mk_aotensor(M) if M is not None else T2(0, [0, 0], [0, 0], cast_dtype(q.dtype))
     params.Out = mk_aotensor(o)
     params.dropout_p = float(dropout_p)
     params.philox_seed_ptr = mk_aotensor(philox_seed)

@@ -5,6 +5,7 @@ import ctypes
 
 from ... import _lib
 from ..._lib import lib
+from .. import DType, T0, T1, T2, T4, hipError_t    # defined before the parent package imports this module
 
 
 class attn_options:
@@ -20,11 +21,17 @@ class attn_options:
 
 
 def _null(cls_name):
-    from .. import T0, T1, T2, T4, DType
-    cls = {'T0': T0, 'T1': T1, 'T2': T2, 'T4': T4}[cls_name]
-    if cls is T0:
-        return T0(0, DType.kUnknown)
-    return cls(0, [0] * cls.RANK, [0] * cls.RANK, DType.kUnknown)
+    """A null view of the given rank.  Views are immutable, so one object per rank serves
+    every params struct."""
+    v = _NULLS.get(cls_name)
+    if v is None:
+        cls = {'T0': T0, 'T1': T1, 'T2': T2, 'T4': T4}[cls_name]
+        v = T0(0, DType.kUnknown) if cls is T0 else cls(0, [0] * cls.RANK, [0] * cls.RANK, DType.kUnknown)
+        _NULLS[cls_name] = v
+    return v
+
+
+_NULLS = {}
 
 
 class attn_fwd_params:
@@ -116,14 +123,12 @@ def _opt(options):
 
 
 def attn_fwd(params, params_version, stream, options=None):
-    from .. import hipError_t
     c = params.to_c()
     keep, optp = _opt(options)
     return hipError_t(lib.fa_attn_fwd(ctypes.byref(c), int(params_version), stream.native() or None, optp))
 
 
 def attn_bwd(params, params_version, stream, options=None):
-    from .. import hipError_t
     c = params.to_c()
     keep, optp = _opt(options)
     return hipError_t(lib.fa_attn_bwd(ctypes.byref(c), int(params_version), stream.native() or None, optp))
@@ -131,28 +136,24 @@ def attn_bwd(params, params_version, stream, options=None):
 
 def attn_bwd_kernel(params, params_version, stream, kernel_slot):
     """Launch one backward kernel only (0 delta, 1 dK/dV, 2 dQ, 3 fused)."""
-    from .. import hipError_t
     c = params.to_c()
     return hipError_t(lib.fa_attn_bwd_kernel(ctypes.byref(c), int(params_version),
                                              stream.native() or None, int(kernel_slot)))
 
 
 def validate_fwd(params, params_version, options=None):
-    from .. import hipError_t
     c = params.to_c()
     keep, optp = _opt(options)
     return hipError_t(lib.fa_validate_fwd(ctypes.byref(c), int(params_version), optp))
 
 
 def validate_bwd(params, params_version, options=None):
-    from .. import hipError_t
     c = params.to_c()
     keep, optp = _opt(options)
     return hipError_t(lib.fa_validate_bwd(ctypes.byref(c), int(params_version), optp))
 
 
 def query_fwd_config(params, num_cu=256):
-    from .. import hipError_t
     c = params.to_c()
     out = _lib.fa_kernel_config()
     err = hipError_t(lib.fa_query_fwd_config(ctypes.byref(c), int(num_cu), ctypes.byref(out)))
@@ -160,7 +161,6 @@ def query_fwd_config(params, num_cu=256):
 
 
 def query_bwd_config(params, kernel_slot, options=None):
-    from .. import hipError_t
     c = params.to_c()
     keep, optp = _opt(options)
     out = _lib.fa_kernel_config()
