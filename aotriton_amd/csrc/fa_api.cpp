@@ -74,6 +74,8 @@ bool is_16bit(int dt) { return dt == FA_DTYPE_FLOAT16 || dt == FA_DTYPE_BFLOAT16
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+constexpr int64_t kMaxRowStride = 1 << 21;   // elements; 256 rows of it stay below 2^31 bytes at 4 bytes per element
+
 // rank-4 activation tensor: non-null unless it has no element, unit last stride, 16-byte aligned rows
 int check_act(const fa_tensor4& t, int dtype) {
   const bool empty = (t.sizes[0] == 0 || t.sizes[1] == 0 || t.sizes[2] == 0) && t.sizes[3] > 0;
@@ -82,7 +84,9 @@ int check_act(const fa_tensor4& t, int dtype) {
   if (t.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
   if (!aligned16(t.ptr)) return FA_ERROR_NOT_SUPPORTED;
   for (int i = 0; i < 3; ++i)
-    if (t.sizes[i] > 1 && (t.strides[i] % 8) != 0) return FA_ERROR_NOT_SUPPORTED;
+    if (t.sizes[i] > 1 && ((t.strides[i] % 8) != 0 || t.strides[i] < 0)) return FA_ERROR_NOT_SUPPORTED;
+  // a tile's rows are addressed with 32-bit byte offsets from the tile's first row
+  if (t.sizes[2] > 1 && t.strides[2] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
   return FA_SUCCESS;
 }
 
@@ -159,6 +163,9 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
     if ((int)B.sizes[0] != s.batch || (int)B.sizes[1] != s.hq || (int)B.sizes[2] != s.max_sq ||
         (int)B.sizes[3] != s.max_sk)
       return FA_ERROR_INVALID_VALUE;
+    for (int i = 0; i < 4; ++i)
+      if (B.strides[i] < 0) return FA_ERROR_NOT_SUPPORTED;
+    if (B.strides[2] > kMaxRowStride * 8 || B.strides[3] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
   }
   *out = s;
   return FA_SUCCESS;
@@ -240,7 +247,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
     if (!s.bias) return FA_ERROR_INVALID_VALUE;
     if (p->DB.dtype != dt) return FA_ERROR_INVALID_VALUE;
     for (int i = 0; i < 4; ++i)
-      if (p->DB.sizes[i] != p->B.sizes[i]) return FA_ERROR_INVALID_VALUE;
+      if (p->DB.sizes[i] != p->B.sizes[i] || p->DB.strides[i] < 0) return FA_ERROR_INVALID_VALUE;
   }
   int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2

@@ -280,6 +280,51 @@ def test_headline_size_properties():
         assert (colsum - dosum).abs().max().item() < 0.5, (colsum - dosum).abs().max().item()
 
 
+def test_tensors_with_more_than_2g_elements():
+    """B520 H64 S1024 D64 bf16 causal: 2,181,038,080 elements per tensor, so element offsets
+    pass 2^31.  Row 0 of every head attends only to key 0 (O[0] == V[0]); the first, a
+    middle and the last head match the oracle; sum_n dV[n] == sum_m dO[m] for every head."""
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    B, H, S, D = 520, 64, 1024, 64
+    assert B * H * S * D > 2 ** 31
+    g = torch.Generator(device=DEV).manual_seed(77)
+    mk = lambda: torch.randn(B, H, S, D, generator=g, device=DEV, dtype=torch.bfloat16)
+    q, k, v, do = mk(), mk(), mk(), mk()
+    sm = 1.0 / math.sqrt(D)
+    for backend in (0, 1):
+        q.grad = k.grad = v.grad = None
+        q.requires_grad_(); k.requires_grad_(); v.requires_grad_()
+        o, _, L = attention(q, k, v, None, True, sm, 0.0,
+                            AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend))
+        o.backward(do)
+        torch.cuda.synchronize()
+        assert torch.equal(o[:, :, 0], v[:, :, 0])
+        assert not bool(torch.isnan(o).any()) and not bool(torch.isnan(L).any())
+        for t in (q.grad, k.grad, v.grad):
+            assert not bool(torch.isnan(t).any())
+        for (b, h) in [(0, 0), (263, 31), (B - 1, H - 1)]:
+            sl = lambda t: t.detach()[b:b + 1, h:h + 1]
+            ro, rl, _ = fa_ref.attn_fwd_ref(sl(q).float(), sl(k).float(), sl(v).float(), None, sm, 3, -2147483647, -2147483647)
+            lo, ll, _ = fa_ref.attn_fwd_ref(sl(q), sl(k), sl(v), None, sm, 3, -2147483647, -2147483647)
+            check('out', sl(o), ro, lo, FUDGE['out'])
+            assert (L.view(B, H, S)[b, h] - rl[0, 0]).abs().max().item() <= LSE_ATOL
+            rg = fa_ref.attn_bwd_ref(sl(q).float(), sl(k).float(), sl(v).float(), None, sm, ro, sl(do).float(), rl,
+                                     3, -2147483647, -2147483647)
+            lg = fa_ref.attn_bwd_ref(sl(q), sl(k), sl(v), None, sm, lo, sl(do), ll.to(torch.bfloat16), 3,
+                                     -2147483647, -2147483647)
+            check('dq', sl(q.grad), rg[0], lg[0], FUDGE['dq'])
+            check('dk', sl(k.grad), rg[1], lg[1], FUDGE['dk'])
+            check('dv', sl(v.grad), rg[2], lg[2], FUDGE['dv'])
+        colsum = v.grad.float().sum(dim=2)
+        dosum = do.float().sum(dim=2)
+        assert (colsum - dosum).abs().max().item() < 0.5, (colsum - dosum).abs().max().item()
+        del o, L, colsum, dosum
+    q.grad = k.grad = v.grad = None
+    del q, k, v, do
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize('layout', ['padded', 'strided'])
 @pytest.mark.parametrize('causal', [False, True])
 @pytest.mark.parametrize('backend', [0, 1])

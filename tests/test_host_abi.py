@@ -126,6 +126,11 @@ def test_validate_fwd_error_contract():
     p.Q = T4(0, [0] * 4, [0] * 4, DType.kBFloat16)
     assert validate_fwd(p, 3) == E.hipErrorInvalidValue                        # null Q
     p, keep = _fwd_params()
+    p.K = T4(p.K.data_ptr, p.K.sizes, [p.K.stride(0), p.K.stride(1), 1 << 22, 1], p.K.dtype)
+    assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # row stride beyond 32-bit tile offsets
+    p.K = T4(p.K.data_ptr, p.K.sizes, [p.K.stride(0), p.K.stride(1), -128, 1], p.K.dtype)
+    assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # negative stride
+    p, keep = _fwd_params()
     p.causal_type = 1
     assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # only 0 and 3 exist
     p.causal_type = 3
