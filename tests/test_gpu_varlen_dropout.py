@@ -280,6 +280,46 @@ def test_headline_size_properties():
         assert (colsum - dosum).abs().max().item() < 0.5, (colsum - dosum).abs().max().item()
 
 
+@pytest.mark.parametrize('backend', [0, 1])
+def test_sequence_of_100k_tokens(backend):
+    """B1 Hq4 Hkv2 S100003 D128 bf16 causal.  Blocks of query rows are compared with the
+    oracle run on those rows against the keys they see (bottom-right aligned causal mask of
+    the slice = the rows' causal mask); the last block's dK/dV rows are complete from the
+    last block of queries alone; sum_n dV[n] == sum_m dO[m]."""
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    B, Hq, Hk, S, D = 1, 4, 2, 100003, 128
+    g = torch.Generator(device=DEV).manual_seed(78)
+    mk = lambda H: torch.randn(B, H, S, D, generator=g, device=DEV, dtype=torch.bfloat16)
+    q, k, v, do = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+    sm = 1.0 / math.sqrt(D)
+    qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+    o, _, L = attention(qg, kg, vg, None, True, sm, 0.0,
+                        AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend))
+    o.backward(do)
+    torch.cuda.synchronize()
+    for t in (o, L, qg.grad, kg.grad, vg.grad):
+        assert not bool(torch.isnan(t).any())
+    BR = -2147483646
+    for i0, i1 in [(0, 64), (65500, 65600), (S - 64, S)]:
+        qs, dos = q[:, :, i0:i1], do[:, :, i0:i1]
+        ks, vs = k[:, :, :i1], v[:, :, :i1]
+        f = lambda t: t.float()
+        ro, rl, _ = fa_ref.attn_fwd_ref(f(qs), f(ks), f(vs), None, sm, 3, BR, BR)
+        lo, ll, _ = fa_ref.attn_fwd_ref(qs, ks, vs, None, sm, 3, BR, BR)
+        check('out', o[:, :, i0:i1], ro, lo, FUDGE['out'])
+        assert (L.view(B, Hq, S)[:, :, i0:i1] - rl).abs().max().item() <= LSE_ATOL
+        rg = fa_ref.attn_bwd_ref(f(qs), f(ks), f(vs), None, sm, ro, f(dos), rl, 3, BR, BR)
+        lg = fa_ref.attn_bwd_ref(qs, ks, vs, None, sm, lo, dos, ll.to(torch.bfloat16), 3, BR, BR)
+        check('dq', qg.grad[:, :, i0:i1], rg[0], lg[0], FUDGE['dq'])
+        if i1 == S:
+            check('dk', kg.grad[:, :, i0:], rg[1][:, :, i0:], lg[1][:, :, i0:], FUDGE['dk'])
+            check('dv', vg.grad[:, :, i0:], rg[2][:, :, i0:], lg[2][:, :, i0:], FUDGE['dv'])
+    colsum = vg.grad.float().sum(dim=2)                                  # (B, Hk, D)
+    dosum = do.float().view(B, Hk, Hq // Hk, S, D).sum(dim=(2, 3))
+    assert (colsum - dosum).abs().max().item() < 1.0, (colsum - dosum).abs().max().item()
+
+
 def test_tensors_with_more_than_2g_elements():
     """B520 H64 S1024 D64 bf16 causal: 2,181,038,080 elements per tensor, so element offsets
     pass 2^31.  Row 0 of every head attends only to key 0 (O[0] == V[0]); the first, a
