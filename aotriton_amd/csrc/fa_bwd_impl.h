@@ -227,6 +227,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   const T* bb = nullptr;
   const T* bb_tile = nullptr;     // bias tile being fetched, its valid rows
   int b_rows = 0;
+  const int b_cols = si.seqlen_k - n0 < BN ? si.seqlen_k - n0 : BN;      // valid keys of this item
   // (g, e) = (q-head inside the GQA group, Q tile inside the range) of the tile to fetch;
   // called for consecutive tiles only; `live` false: nothing is fetched
   auto fetch_begin = [&](bool live, int g, int e) {
@@ -241,9 +242,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
              (int64_t)(hk * group + g) * a.sb_h + (int64_t)br.lo * BM * a.sb_m + (int64_t)n0 * a.sb_n;
       bb_tile = bb;
       b_rows = rows;
-      const int cols = si.seqlen_k - n0 < BN ? si.seqlen_k - n0 : BN;
       b_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(bb), 0,
-                                               any && bias_lds ? ((rows - 1) * (int)a.sb_m + cols) * 2 : 0, 0x00020000);
+                                               any && bias_lds ? ((rows - 1) * (int)a.sb_m + b_cols) * 2 : 0, 0x00020000);
       if (live) bb += (int64_t)BM * a.sb_m;
     }
     q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0,
@@ -269,6 +269,18 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       const int k = i - 2 * CH;
       if (bias_lds) {
         bch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_voff, k * b_soff, 0));
+        // The descriptor ends at the last valid element of the tile's last row.  When that is
+        // not at a 16-byte boundary the piece that straddles the end loses its valid elements
+        // to the range check too (a dword that holds the last of an odd number of columns reads
+        // as zero): that one piece is gathered element by element.
+        const int row = tid / 16 + k * (NT / 16), col = (tid % 16) * 8;
+        if ((b_cols & 7) != 0 && row == b_rows - 1 && col < b_cols && col + 8 > b_cols) {
+          op_t x;
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            x[e] = col + e < b_cols ? bb_tile[(int64_t)row * a.sb_m + col + e] : Tr::cvt(0.f);
+          bch[k] = x;
+        }
       } else {
         // any other layout: the piece is gathered element by element
         const int row = tid / 16 + k * (NT / 16), col = (tid % 16) * 8;

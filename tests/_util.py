@@ -3,9 +3,11 @@ tolerance model (modules/flash/tests/_common_test.py:459-495):
     max|out - ref_hp| <= max(1e-5, fudge * max|ref_hp - ref_lp|)
 with ref_hp the oracle in fp32 and ref_lp the oracle in the input dtype (fp64 and fp32
 for fp32 inputs, _common_test.py:347).
-Fudge factors: out 3.0, dq 148, dk 48, dv 36, db 17 (_common_test.py:171-180,384-407).
+Fudge factors: out 3.0, dq 148, dk 48, dv 36, db 17 (_common_test.py:171-180,384-407),
+each capped at STRICT_FACTOR here.
 """
 import math
+import os
 
 import numpy as np
 import torch
@@ -16,6 +18,7 @@ FUDGE = dict(out=3.0, dq=148.0, dk=48.0, dv=36.0, db=17.0)
 # the LSE has no entry in the reference's tolerance table (its tests only check
 # the known-answer case); fp32 accumulation of 16-bit products, absolute bound
 LSE_ATOL = 2e-3
+STRICT_FACTOR = 6.0
 
 
 def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False, bias_layout='padded',
@@ -61,6 +64,14 @@ def check(name, out, ref_hp, ref_lp, fudge, mask=None):
     assert not torch.isnan(out).any(), f'{name}: NaN in output'
     err = (out - ref_hp).abs().max().item() if out.numel() else 0.0
     ref_err = (ref_lp - ref_hp).abs().max().item() if out.numel() else 0.0
-    thr = max(1e-5, fudge * ref_err)
+    # The reference's factors are what its own kernels need on their worst shapes; with
+    # dk 48, dv 36 or dq 148 a wrong element can hide (a bias value read as zero for one key
+    # of one row per tile did, at 8x the 16-bit oracle's error).  These kernels stay within
+    # 4.3x of the low-precision oracle's error over the whole suite, so they are held to 6x.
+    thr = max(1e-5, min(fudge, STRICT_FACTOR) * ref_err)
+    log = os.environ.get('FA_TEST_ERROR_LOG')
+    if log:      # one line per checked tensor: error relative to the low-precision oracle's
+        with open(log, 'a') as f:
+            f.write(f"{os.environ.get('PYTEST_CURRENT_TEST', '?')}\t{name}\t{err:.4e}\t{ref_err:.4e}\n")
     assert err <= thr, f'{name}: max|out-ref|={err:.3e} > {thr:.3e} (ref_lp err {ref_err:.3e}, fudge {fudge})'
     return err, thr

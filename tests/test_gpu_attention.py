@@ -163,6 +163,66 @@ def test_fp32_has_no_fused_backend():
         o.backward(do)
 
 
+def _sampled_grid_cases(n=72, seed=2024):
+    """A seeded sample of the reference's test grids (tests/test_backward.py:35-142 with the
+    lists of tests/_core_test_backward.py:60-89): regular, matrix bias, GQA, irregular
+    (prime) sequence lengths and Dqk != Dv, over all dtypes, both storage orders, both
+    scales and both backward backends.  Sequence lengths above 2048 are left out and a
+    dropout case keeps Sq*Sk small (its mask comes from the CPU oracle)."""
+    import random
+    rnd = random.Random(seed)
+    hd_all = sorted(set([16, 32, 64, 128, 256, 512, 48, 80, 96, 160, 192, 224,
+                         8, 24, 40, 56, 72, 88, 96, 120, 152, 184, 216, 248, 408]))
+    regular = [8, 16, 32, 64, 128, 256, 512, 1024, 2048]
+    prime_q = [11, 17, 37, 67, 157, 257, 523, 1033]
+    prime_k = [13, 31, 41, 71, 223, 337, 571, 1063]
+    cases = []
+    for i in range(n):
+        fam = ['regular', 'bias', 'gqa', 'irregular', 'qk_ne_vo'][i % 5]
+        dtype = rnd.choice([torch.float16, torch.bfloat16, torch.float32])
+        D = rnd.choice(hd_all); Dv = None
+        heads = (5, 5); bias = False; flip = rnd.random() < 0.5
+        causal = rnd.random() < 0.5
+        scale = rnd.choice(['l1', 'l2'])
+        if fam == 'regular':
+            sq, sk = rnd.choice(regular), rnd.choice(regular)
+        elif fam == 'bias':
+            sq, sk = rnd.choice(regular), rnd.choice(regular); bias = True; causal = False; scale = 'l1'
+        elif fam == 'gqa':
+            heads = rnd.choice([(16, 8), (10, 2)]); flip = False
+            sq, sk = rnd.choice([4, 143, 2048]), rnd.choice([4, 127, 579, 2048])
+        elif fam == 'irregular':
+            sq, sk = rnd.choice(prime_q), rnd.choice(prime_k); bias = rnd.random() < 0.5
+        else:
+            sq, sk = rnd.choice(prime_q[:7]), rnd.choice(prime_k[:7]); bias = rnd.random() < 0.5
+            Dv = rnd.choice(hd_all); flip = False; scale = 'l1'
+        if bias:
+            causal = False          # the reference skips causal with an explicit bias
+        p = rnd.choice([0.0, 0.5])
+        if p > 0.0 and sq * sk > 600 * 600:
+            p = 0.0
+        if max(D, Dv or 0) > 256 and sq * sk > 1024 * 1024:
+            sq, sk = min(sq, 512), min(sk, 512)      # vector-ALU kernels: keep the case short
+        split_only = dtype == torch.float32 or max(D, Dv or 0) > 256
+        backend = 0 if split_only else rnd.choice([0, 1])
+        cases.append((fam, heads, D, Dv, sq, sk, causal, p, dtype, flip, bias, scale, backend))
+    return cases
+
+
+def _case_id(c):
+    fam, heads, D, Dv, sq, sk, causal, p, dtype, flip, bias, scale, backend = c
+    return (f"{fam}-h{heads[0]}_{heads[1]}-d{D}{'_%d' % Dv if Dv else ''}-q{sq}-k{sk}-{'c' if causal else 'n'}"
+            f"-p{p}-{str(dtype)[6:]}-{'bshd' if flip else 'bhsd'}-{'bias' if bias else 'nobias'}-{scale}-be{backend}")
+
+
+@pytest.mark.parametrize('case', _sampled_grid_cases(), ids=_case_id)
+def test_sample_of_the_reference_grids(case):
+    fam, heads, D, Dv, sq, sk, causal, p, dtype, flip, bias, scale, backend = case
+    sm = 1.0 / D if scale == 'l1' else 1.0 / math.sqrt(D)
+    _run_case(3, heads[0], heads[1], sq, sk, D, dtype, causal, dropout_p=p, bias=bias, bshd=flip,
+              bwd_backend=backend, sm_scale=sm, seed=20, Dv=Dv)
+
+
 @pytest.mark.parametrize('causal', [1, 2])
 def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
     # rows with no visible key: O = 0, LSE = +inf, gradients finite
