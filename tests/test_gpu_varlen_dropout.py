@@ -55,34 +55,30 @@ def test_compact_varlen_gqa(dtype, D, causal, backend):
     check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
 
 
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize('causal', [False, True])
-@pytest.mark.parametrize('backend', [0, 1])
-def test_compact_varlen_with_empty_sequences(dtype, causal, backend):
-    # sequences without queries, without keys and without both among ordinary ones, and
-    # query and key lengths that differ: rows without a key give O = 0, LSE = +inf, dQ = 0;
-    # keys without a query give dK = dV = 0
+def _run_varlen_case(lq, lk, Hq, Hk, D, dtype, causal, backend, p=0.0, seed=11):
+    """Packed sequences against the dense oracle, sequence by sequence.  Rows without a key
+    give O = 0, LSE = +inf, dQ = 0; keys without a query give dK = dV = 0."""
     from aotriton_amd import flash
     from aotriton_amd.autograd import attention_varlen, AttentionExtraArgs
-    from oracle import fa_ref
-    if dtype == torch.float32 and backend == 1:
-        pytest.skip('fp32 has the split backend only')
-    lq = np.array([5, 0, 70, 0, 33, 130])
-    lk = np.array([9, 64, 0, 0, 33, 40])
-    Hq, Hk, D = 4, 2, 64
+    from oracle import fa_ref, philox
+    lq, lk = np.asarray(lq), np.asarray(lk)
     cq = [0] + np.cumsum(lq).tolist()
     ck = [0] + np.cumsum(lk).tolist()
-    g = torch.Generator().manual_seed(11)
+    g = torch.Generator().manual_seed(seed)
     mk = lambda H, T: torch.randn(1, T, H, D, generator=g).to(dtype).to(DEV).transpose(1, 2)
     q, do = mk(Hq, cq[-1]), mk(Hq, cq[-1])
     k, v = mk(Hk, ck[-1]), mk(Hk, ck[-1])
     sm = 1.0 / math.sqrt(D)
     qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
     ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=backend)
-    o, _, L = attention_varlen(qg, kg, vg, lq, lk, causal, sm, 0.0, ext)
+    o, _, L = attention_varlen(qg, kg, vg, lq, lk, causal, sm, p, ext)
     o.backward(do)
     torch.cuda.synchronize()
     ct, wl, wr = flash.translate_causal(causal)
+    keep = None
+    if p > 0.0:      # counters use the sequence index and the maximal lengths (fwd_kernel.py:405-407)
+        keep = philox.dropout_keep_mask(len(lq), Hq, int(lq.max()), int(lk.max()), p, ext.philox_seed,
+                                        ext.philox_offset1 + ext.philox_offset2)
     hp = torch.float64 if dtype == torch.float32 else torch.float32
     f = lambda t: t.to(hp)
     for i in range(len(lq)):
@@ -94,21 +90,73 @@ def test_compact_varlen_with_empty_sequences(dtype, causal, backend):
             assert torch.count_nonzero(o[:, :, sq]) == 0 and bool(torch.isposinf(L[:, sq]).all())
             assert torch.count_nonzero(qg.grad[:, :, sq]) == 0
             continue
-        ro, rl, _ = fa_ref.attn_fwd_ref(f(q[:, :, sq]), f(k[:, :, sk]), f(v[:, :, sk]), None, sm, ct, wl, wr)
-        lo, ll, _ = fa_ref.attn_fwd_ref(q[:, :, sq], k[:, :, sk], v[:, :, sk], None, sm, ct, wl, wr)
+        km = None if keep is None else torch.from_numpy(keep[i:i + 1, :, :lq[i], :lk[i]]).to(DEV)
+        ro, rl, _ = fa_ref.attn_fwd_ref(f(q[:, :, sq]), f(k[:, :, sk]), f(v[:, :, sk]), None, sm, ct, wl, wr, p, km)
+        lo, ll, _ = fa_ref.attn_fwd_ref(q[:, :, sq], k[:, :, sk], v[:, :, sk], None, sm, ct, wl, wr, p, km)
         check(f'out[{i}]', o[:, :, sq], ro, lo, FUDGE['out'])
         live = torch.isfinite(rl[0])
         assert torch.equal(torch.isinf(L[:, sq]), ~live)
-        assert (L[:, sq][live] - rl[0][live]).abs().max().item() <= LSE_ATOL
+        assert not bool(live.any()) or (L[:, sq][live] - rl[0][live]).abs().max().item() <= LSE_ATOL
         rg = fa_ref.attn_bwd_ref(f(q[:, :, sq]), f(k[:, :, sk]), f(v[:, :, sk]), None, sm, ro, f(do[:, :, sq]), rl,
-                                 ct, wl, wr)
+                                 ct, wl, wr, p, km)
         lg = fa_ref.attn_bwd_ref(q[:, :, sq], k[:, :, sk], v[:, :, sk], None, sm, lo, do[:, :, sq],
-                                 ll.to(dtype), ct, wl, wr)
+                                 ll.to(dtype), ct, wl, wr, p, km)
         check(f'dq[{i}]', qg.grad[:, :, sq], rg[0], lg[0], FUDGE['dq'])
         check(f'dk[{i}]', kg.grad[:, :, sk], rg[1], lg[1], FUDGE['dk'])
         check(f'dv[{i}]', vg.grad[:, :, sk], rg[2], lg[2], FUDGE['dv'])
-    assert not bool(torch.isnan(o).any()) and not bool(torch.isnan(qg.grad).any())
-    assert not bool(torch.isnan(kg.grad).any()) and not bool(torch.isnan(vg.grad).any())
+    for t in (o, qg.grad, kg.grad, vg.grad):
+        assert not bool(torch.isnan(t).any())
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('causal', [False, True])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_compact_varlen_with_empty_sequences(dtype, causal, backend):
+    # sequences without queries, without keys and without both among ordinary ones, and
+    # query and key lengths that differ
+    if dtype == torch.float32 and backend == 1:
+        pytest.skip('fp32 has the split backend only')
+    _run_varlen_case([5, 0, 70, 0, 33, 130], [9, 64, 0, 0, 33, 40], 4, 2, 64, dtype, causal, backend)
+
+
+def _sampled_varlen_cases(n=40, seed=4242):
+    """Seeded packed-sequence cases: 1-6 sequences of 0-300 tokens (the reference draws its
+    lengths from a fixed list, tests/test_varlen.py:34-47), key lengths that differ from the
+    query lengths in a third of the cases, GQA, head dims of the reference's list, dropout,
+    windows and both alignments."""
+    import random
+    from aotriton_amd.flash import CausalType
+    rnd = random.Random(seed)
+    cases = []
+    for i in range(n):
+        ns = rnd.randint(1, 6)
+        pick = lambda: rnd.choice([0, 1, 4, 8, 63, 64, 65, 128, 143, 257, 301])
+        lq = [pick() for _ in range(ns)]
+        lk = [pick() for _ in range(ns)] if rnd.random() < 0.33 else list(lq)
+        if sum(lq) == 0: lq[0] = 17
+        if sum(lk) == 0: lk[0] = 17
+        Hq, Hk = rnd.choice([(4, 4), (8, 2), (6, 1), (2, 2)])
+        D = rnd.choice([16, 40, 64, 96, 128, 192, 256, 408])
+        dtype = rnd.choice([torch.float16, torch.bfloat16, torch.float32])
+        r = rnd.random()
+        causal = False if r < 0.3 else (True if r < 0.6 else
+                                        ((rnd.randint(-3, 200), rnd.randint(-3, 200)) if r < 0.8 else CausalType.BOTTOM_RIGHT))
+        p = rnd.choice([0.0, 0.0, 0.3])
+        if p > 0.0:
+            # With a single key dS = P (dP - delta) is exactly zero, and the low-precision oracle
+            # rounds dP and delta alike, so its error (the yardstick) is ~0, while a kernel that
+            # takes delta from the rounded O keeps that rounding in dQ.  Two keys avoid the case.
+            lq = [2 if x == 1 else x for x in lq]
+            lk = [2 if x == 1 else x for x in lk]
+        backend = 0 if (dtype == torch.float32 or D > 256) else rnd.choice([0, 1])
+        cases.append((tuple(lq), tuple(lk), Hq, Hk, D, dtype, causal, backend, p))
+    return cases
+
+
+@pytest.mark.parametrize('case', _sampled_varlen_cases(), ids=lambda c: f"n{len(c[0])}-h{c[2]}_{c[3]}-d{c[4]}-{str(c[5])[6:]}-be{c[7]}-p{c[8]}")
+def test_sampled_packed_sequences(case):
+    lq, lk, Hq, Hk, D, dtype, causal, backend, p = case
+    _run_varlen_case(lq, lk, Hq, Hk, D, dtype, causal, backend, p)
 
 
 def test_compact_varlen_fp32():
@@ -369,14 +417,41 @@ def test_tensors_with_more_than_2g_elements():
 @pytest.mark.parametrize('causal', [False, True])
 @pytest.mark.parametrize('backend', [0, 1])
 def test_padded_and_strided_varlen(layout, causal, backend):
+    _run_layout_case(layout, causal, backend, [70, 5, 192, 133], [3, 11, 0, 60], 128, torch.bfloat16, 4, 2)
+
+
+def _sampled_layout_cases(n=24, seed=77):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    for i in range(n):
+        ns = rnd.randint(1, 5)
+        lens = [rnd.choice([0, 2, 5, 31, 64, 70, 129, 192, 260]) for _ in range(ns)]
+        if max(lens) == 0: lens[0] = 9
+        pads = [rnd.choice([0, 0, 3, 8, 60]) for _ in range(ns)]
+        D = rnd.choice([32, 64, 72, 128, 256, 320])
+        dtype = rnd.choice([torch.float16, torch.bfloat16, torch.float32])
+        Hq, Hk = rnd.choice([(4, 2), (3, 3), (8, 1)])
+        causal = rnd.choice([False, True])
+        backend = 0 if (dtype == torch.float32 or D > 256) else rnd.choice([0, 1])
+        cases.append((['padded', 'strided'][i % 2], causal, backend, tuple(lens), tuple(pads), D, dtype, Hq, Hk))
+    return cases
+
+
+@pytest.mark.parametrize('case', _sampled_layout_cases(),
+                         ids=lambda c: f"{c[0]}-{'c' if c[1] else 'n'}-be{c[2]}-n{len(c[3])}-d{c[5]}-{str(c[6])[6:]}-h{c[7]}_{c[8]}")
+def test_sampled_padded_and_strided_varlen(case):
+    _run_layout_case(*case)
+
+
+def _run_layout_case(layout, causal, backend, lens, pads, D, dtype, Hq, Hk):
     # varlen_type 2: rank-4 batch tensors padded to the longest sequence, LSE (n*Hq, max_sq);
     # varlen_type 3: packed tokens with gaps, sequence starts from seq_strides, LSE (Hq, total)
     # (modules/flash/kernel/fwd_kernel.py:243-286, tests/varlen_attn_torch_function.py:52-84).
     from aotriton_amd import flash
     from oracle import fa_ref
-    dtype, D, Hq, Hk = torch.bfloat16, 128, 4, 2
-    lens = np.array([70, 5, 192, 133])
-    pads = np.array([3, 11, 0, 60])
+    lens = np.asarray(lens)
+    pads = np.asarray(pads)
     n, mx = len(lens), int(lens.max())
     g = torch.Generator().manual_seed(11)
     rn = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)
@@ -408,8 +483,11 @@ def test_padded_and_strided_varlen(layout, causal, backend):
                                  0.0, null, null, 0, causal, layout, extargs=ext) == ok
     torch.cuda.synchronize()
     ct, wl, wr = flash.translate_causal(causal)
-    f = lambda t: t.float()
+    hp = torch.float64 if dtype == torch.float32 else torch.float32
+    f = lambda t: t.to(hp)
     for i in range(n):
+        if lens[i] == 0:
+            continue
         qi, ki, vi, doi = sl(q, i), sl(k, i), sl(v, i), sl(do, i)
         ro, rl, _ = fa_ref.attn_fwd_ref(f(qi), f(ki), f(vi), None, sm, ct, wl, wr, 0.0, None)
         lo, ll, _ = fa_ref.attn_fwd_ref(qi, ki, vi, None, sm, ct, wl, wr, 0.0, None)
@@ -422,10 +500,14 @@ def test_padded_and_strided_varlen(layout, causal, backend):
         check(f'dk[{i}]', sl(dk, i), rg[1], lg[1], FUDGE['dk'])
         check(f'dv[{i}]', sl(dv, i), rg[2], lg[2], FUDGE['dv'])
     # rows outside the sequences are never written
-    if layout == 'padded':
-        assert torch.isnan(o[1, :, lens[1]:]).all() and torch.isnan(dk[1, :, lens[1]:]).all()
-    else:
-        assert torch.isnan(o[:, :, lens[0]:starts[1]]).all() and torch.isnan(dv[:, :, lens[0]:starts[1]]).all()
+    for i in range(n):
+        if layout == 'padded':
+            assert torch.isnan(o[i, :, lens[i]:]).all() and torch.isnan(dk[i, :, lens[i]:]).all()
+            assert torch.isnan(dq[i, :, lens[i]:]).all() and torch.isnan(dv[i, :, lens[i]:]).all()
+        else:
+            gap = slice(starts[i] + lens[i], starts[i + 1])
+            assert torch.isnan(o[:, :, gap]).all() and torch.isnan(dv[:, :, gap]).all()
+            assert torch.isnan(dq[:, :, gap]).all() and torch.isnan(dk[:, :, gap]).all()
 
 
 def test_config4_full_size_properties():
