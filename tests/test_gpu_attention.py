@@ -223,6 +223,87 @@ def test_sample_of_the_reference_grids(case):
               bwd_backend=backend, sm_scale=sm, seed=20, Dv=Dv)
 
 
+def _layout_case(i, seed=3):
+    import random
+    from aotriton_amd.flash import CausalType
+    rnd = random.Random(seed * 100003 + i)
+    c = dict(i=i)
+    c['B'] = rnd.choice([1, 2, 3]); c['Hk'] = rnd.choice([1, 2, 3]); c['Hq'] = c['Hk'] * rnd.choice([1, 1, 2, 4])
+    c['D'] = rnd.choice([16, 40, 64, 72, 128, 160, 256])
+    c['Dv'] = c['D'] if rnd.random() < 0.8 else rnd.choice([32, 64, 128])
+    lens = [1, 2, 7, 31, 64, 65, 127, 128, 129, 200, 256, 257, 383, 512, 700]
+    c['sq'] = rnd.choice(lens); c['sk'] = rnd.choice(lens)
+    c['dtype'] = rnd.choice([torch.float16, torch.bfloat16, torch.float32])
+    c['layout'] = rnd.choice(['bhsd', 'bshd', 'qkv', 'gap'])
+    c['bias'] = rnd.choice([None, None, 'full', 'odd', 'bcast_b', 'bcast_h', 'bcast_bh', 'bcast_m'])
+    r = rnd.random()
+    c['causal'] = False if r < 0.3 else (True if r < 0.55 else (
+        (rnd.randint(-3, c['sq']), rnd.randint(-3, c['sk'])) if r < 0.8 else CausalType.BOTTOM_RIGHT))
+    c['p'] = rnd.choice([0.0, 0.0, 0.2]) if c['sk'] > 1 else 0.0
+    split_only = c['dtype'] == torch.float32 or max(c['D'], c['Dv']) > 256
+    c['be'] = 0 if split_only else rnd.choice([0, 1])
+    c['sm'] = rnd.choice([1.0 / c['D'], c['D'] ** -0.5])
+    return c
+
+
+@pytest.mark.parametrize('i', range(64))
+def test_sampled_strides_bias_layouts_and_masks(i):
+    """Seeded cases over what the callers' tensors look like: BHSD, BSHD, q/k/v as slices of one
+    packed (B, S, 3, H, D) tensor, rows wider than the head dim; bias padded, with odd row
+    stride, broadcast along batch, heads, both or the query rows; windows, both causal
+    alignments and dropout on top; sequence lengths from 1 to 700."""
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    c = _layout_case(i)
+    B, Hq, Hk, D, Dv, sq, sk, dtype = (c[x] for x in ('B', 'Hq', 'Hk', 'D', 'Dv', 'sq', 'sk', 'dtype'))
+    g = torch.Generator().manual_seed(1000 + i)
+    rn = lambda *s, scale=1.0: (torch.randn(*s, generator=g) * scale).to(dtype).to(DEV)
+    if c['layout'] == 'qkv' and Hq == Hk and D == Dv and sq == sk:
+        qkv = rn(B, sq, 3, Hq, D)
+        q, k, v = [qkv[:, :, j].transpose(1, 2) for j in range(3)]
+    elif c['layout'] == 'bshd':
+        q = rn(B, sq, Hq, D).transpose(1, 2); k = rn(B, sk, Hk, D).transpose(1, 2); v = rn(B, sk, Hk, Dv).transpose(1, 2)
+    elif c['layout'] == 'gap':
+        q = rn(B, Hq, sq, D + 24)[..., 8:8 + D]; k = rn(B, Hk, sk, D + 8)[..., :D]; v = rn(B, Hk, sk, Dv + 16)[..., 16:]
+    else:
+        q = rn(B, Hq, sq, D); k = rn(B, Hk, sk, D); v = rn(B, Hk, sk, Dv)
+    do = rn(B, Hq, sq, Dv)
+    kind, b = c['bias'], None
+    if kind == 'full': b = rn(B, Hq, sq, (sk + 7) // 8 * 8, scale=0.5)[..., :sk]
+    elif kind == 'odd': b = rn(B, Hq, sq, sk + 3, scale=0.5)[..., 1:sk + 1]
+    elif kind == 'bcast_b': b = rn(1, Hq, sq, sk, scale=0.5).expand(B, Hq, sq, sk)
+    elif kind == 'bcast_h': b = rn(B, 1, sq, sk, scale=0.5).expand(B, Hq, sq, sk)
+    elif kind == 'bcast_bh': b = rn(1, 1, sq, sk, scale=0.5).expand(B, Hq, sq, sk)
+    elif kind == 'bcast_m': b = rn(B, Hq, 1, sk, scale=0.5).expand(B, Hq, sq, sk)
+    need_db = kind in ('full', 'odd')
+    causal, p, sm = c['causal'], c['p'], c['sm']
+    ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=c['be'])
+    qg, kg, vg = [t.detach().requires_grad_() for t in (q, k, v)]     # keeps the strides
+    bg = b.detach().requires_grad_() if need_db else b
+    o, _, L = attention(qg, kg, vg, bg, causal, sm, p, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    ct, wl, wr = flash.translate_causal(causal)
+    keep = keep_mask_from_oracle(B, Hq, sq, sk, p, ext.philox_seed, ext.philox_offset1 + ext.philox_offset2, DEV)
+    hp = torch.float64 if dtype == torch.float32 else torch.float32
+    f = lambda t: None if t is None else t.to(hp)
+    ro, rl, _ = fa_ref.attn_fwd_ref(f(q), f(k), f(v), f(b), sm, ct, wl, wr, p, keep)
+    lo, ll, _ = fa_ref.attn_fwd_ref(q, k, v, b, sm, ct, wl, wr, p, keep)
+    live = torch.isfinite(rl)
+    check('out', o, ro, lo, FUDGE['out'])
+    Lv = L.view(B, Hq, sq)
+    assert torch.equal(torch.isinf(Lv), ~live)
+    assert not bool(live.any()) or (Lv[live] - rl[live]).abs().max().item() <= LSE_ATOL
+    rg = fa_ref.attn_bwd_ref(f(q), f(k), f(v), f(b), sm, ro, f(do), rl, ct, wl, wr, p, keep)
+    lg = fa_ref.attn_bwd_ref(q, k, v, b, sm, lo, do, ll.to(q.dtype), ct, wl, wr, p, keep)
+    check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
+    check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
+    check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
+    if need_db:
+        check('db', bg.grad, rg[3], lg[3], FUDGE['db'])
+
+
 @pytest.mark.parametrize('causal', [1, 2])
 def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
     # rows with no visible key: O = 0, LSE = +inf, gradients finite
