@@ -16,7 +16,7 @@ DEV = 'cuda'
 
 
 def _run_case(B, Hq, Hk, Sq, Sk, D, dtype, causal, dropout_p=0.0, bias=False, bshd=False,
-              bwd_backend=-1, sm_scale=None, seed=0, bias_layout='padded', Dv=None):
+              bwd_backend=-1, sm_scale=None, seed=0, bias_layout='padded', Dv=None, philox=None):
     from aotriton_amd import flash
     from aotriton_amd.autograd import attention, AttentionExtraArgs
     from oracle import fa_ref
@@ -24,6 +24,8 @@ def _run_case(B, Hq, Hk, Sq, Sk, D, dtype, causal, dropout_p=0.0, bias=False, bs
                                  bias_layout=bias_layout, Dv=Dv)
     sm_scale = 1.0 / math.sqrt(D) if sm_scale is None else sm_scale
     ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=bwd_backend)
+    if philox is not None:
+        ext.philox_seed, ext.philox_offset1, ext.philox_offset2 = philox
     qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
     bg = b.detach().requires_grad_() if b is not None else None      # keeps the strides of b
     o, _, L = attention(qg, kg, vg, bg, causal, sm_scale, dropout_p, ext)
@@ -78,6 +80,13 @@ def test_ragged_gqa_bshd(dtype, D, sq, sk, causal):
 @pytest.mark.parametrize('backend', [0, 1])
 def test_dropout(D, causal, backend):
     _run_case(2, 5, 5, 197, 223, D, torch.float16, causal, dropout_p=0.5, bwd_backend=backend)
+
+
+@pytest.mark.parametrize('backend', [0, 1])
+def test_dropout_with_64_bit_seed_and_offsets(backend):
+    # forward, dK/dV and dQ kernels must draw the same mask from a seed and offsets that use all 64 bits
+    _run_case(2, 4, 2, 130, 259, 128, torch.bfloat16, True, dropout_p=0.3, bwd_backend=backend,
+              philox=(0xDEADBEEF12345678, (1 << 32) - 2, (1 << 40) + 7))
 
 
 @pytest.mark.parametrize('D', [64, 128, 256])

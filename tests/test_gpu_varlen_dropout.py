@@ -14,7 +14,7 @@ DEV = 'cuda'
 
 
 def _u64(x):
-    return torch.tensor([x], dtype=torch.int64, device=DEV).view(torch.uint64)
+    return torch.tensor([int(np.uint64(x).astype(np.int64))], dtype=torch.int64, device=DEV).view(torch.uint64)
 
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
@@ -215,13 +215,17 @@ def test_varlen_dropout_mask_uses_sequence_index_and_max_seqlens():
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('shape', [(2, 3, 70, 131), (1, 2, 64, 32), (1, 1, 1, 5)])
 @pytest.mark.parametrize('p', [0.1, 0.5])
-def test_encoded_softmax_is_bit_exact(dtype, shape, p):
+@pytest.mark.parametrize('state', [(0x1234, (1 << 32) - 3, 9), (0xDEADBEEF12345678, 0x100000005, (1 << 40) + 7),
+                                   ((1 << 64) - 1, (1 << 63) + 11, (1 << 63) - 5)], ids=['carry', 'wide', 'wrap'])
+def test_encoded_softmax_is_bit_exact(dtype, shape, p, state):
+    # seeds and offsets that use all 64 bits; a counter that carries into its high word, and
+    # offset1 + offset2 that wraps around 2^64
     from aotriton_amd import flash
     from oracle import philox
     B, H, Sq, Sk = shape
     sk8 = (Sk + 7) // 8 * 8
     r = torch.zeros(B, H, Sq, sk8, dtype=dtype, device=DEV)[..., :Sk]
-    seed, off1, off2 = 0x1234, (1 << 32) - 3, 9
+    seed, off1, off2 = state
     assert flash.debug_simulate_encoded_softmax(r, p, _u64(seed), _u64(off1), off2) == flash.hipError_t.hipSuccess
     torch.cuda.synchronize()
     keep = philox.dropout_keep_mask(B, H, Sq, Sk, p, seed, off1 + off2)
