@@ -90,6 +90,17 @@ int check_act(const fa_tensor4& t, int dtype) {
   return FA_SUCCESS;
 }
 
+// L and delta: fp32, contiguous, one value per (sequence or batch element, query head, query row)
+// in the layout the kernels index ((batch * Hq, max_seqlen_q) for rank-4 batches, (Hq, tokens)
+// for packed sequences; modules/flash/kernel/fwd_kernel_inner.py:38-43).
+int check_row_stats(const fa_tensor2& t, int64_t need) {
+  if (t.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  if (t.sizes[1] > 1 && t.strides[1] != 1) return FA_ERROR_NOT_SUPPORTED;
+  if (t.sizes[0] > 1 && t.strides[0] != (int64_t)t.sizes[1]) return FA_ERROR_NOT_SUPPORTED;
+  if ((int64_t)t.sizes[0] * (int64_t)t.sizes[1] < need) return FA_ERROR_INVALID_VALUE;
+  return FA_SUCCESS;
+}
+
 fa::Strides3 strides3(const fa_tensor4& t) {
   return fa::Strides3{(int64_t)t.strides[0], (int64_t)t.strides[1], (int64_t)t.strides[2]};
 }
@@ -97,6 +108,7 @@ fa::Strides3 strides3(const fa_tensor4& t) {
 struct Shape {
   int batch, hq, hk, d, d_qk, d_v, max_sq, max_sk, num_seqlens;  // d: compiled head dim; d_qk, d_v: the tensors'; num_seqlens signed as in attn_fwd.cc:99
   bool windowed, bias, dropout;
+  int64_t row_stats;      // elements of L and of delta
 };
 
 // Shared by forward and backward: everything that only depends on
@@ -151,6 +163,8 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   } else if (varlen_type != FA_VARLEN_NONE) {
     return FA_ERROR_INVALID_VALUE;
   }
+  s.row_stats = s.num_seqlens > 0 ? (int64_t)s.hq * (int64_t)Q.sizes[2]
+                                  : (int64_t)s.batch * s.hq * (int64_t)s.max_sq;
   if (causal_type != FA_CAUSAL_NONE && causal_type != FA_CAUSAL_WINDOWED) return FA_ERROR_NOT_SUPPORTED;
   s.windowed = causal_type != FA_CAUSAL_NONE;
   if (!(dropout_p >= 0.0f) || !(dropout_p < 1.0f)) return FA_ERROR_INVALID_VALUE;
@@ -197,7 +211,7 @@ int validate_fwd(const fa_fwd_params* p, int32_t version, const fa_options* opt,
   for (int i = 0; i < 4; ++i)
     if (p->Out.sizes[i] != (i == 3 ? p->V.sizes[3] : p->Q.sizes[i])) return FA_ERROR_INVALID_VALUE;
   if (p->A.ptr != nullptr) return FA_ERROR_NOT_SUPPORTED;   // alibi: USE_ALIBI=false in attn_fwd.cc:123
-  if (p->L.ptr != nullptr && p->L.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  if (p->L.ptr != nullptr && (e = check_row_stats(p->L, s.row_stats)) != FA_SUCCESS) return e;
   if (p->encoded_softmax.ptr != nullptr) {
     const fa_tensor4& r = p->encoded_softmax;
     if (r.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
@@ -242,7 +256,8 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   }
   // without a query row L and delta hold nothing and may be null
   const bool no_query = p->Q.sizes[0] == 0 || p->Q.sizes[2] == 0;
-  if ((p->L.ptr == nullptr && !no_query) || p->L.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+  if (p->L.ptr == nullptr && !no_query) return FA_ERROR_INVALID_VALUE;
+  if (p->L.ptr != nullptr && (e = check_row_stats(p->L, s.row_stats)) != FA_SUCCESS) return e;
   if (p->DB.ptr != nullptr) {
     if (!s.bias) return FA_ERROR_INVALID_VALUE;
     if (p->DB.dtype != dt) return FA_ERROR_INVALID_VALUE;
@@ -260,7 +275,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   }
   if (be == 0) {
     if (p->D.eager.ptr == nullptr && p->D.acquire == nullptr) return FA_ERROR_INVALID_VALUE;
-    if (p->D.eager.ptr != nullptr && p->D.eager.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
+    if (p->D.eager.ptr != nullptr && (e = check_row_stats(p->D.eager, s.row_stats)) != FA_SUCCESS) return e;
   }
   if (shape) *shape = s;
   if (backend) *backend = be;
@@ -534,6 +549,10 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
       const bool no_query = p->Q.sizes[0] == 0 || p->Q.sizes[2] == 0;
       if (lazy->acquire(lazy, &delta) != 0 || (delta.ptr == nullptr && !no_query)) return FA_ERROR_INVALID_VALUE;
       acquired = true;
+      if (delta.ptr != nullptr && check_row_stats(delta, s.row_stats) != FA_SUCCESS) {
+        if (lazy->dispose != nullptr) lazy->dispose(lazy);
+        return FA_ERROR_INVALID_VALUE;
+      }
     }
     a.delta = static_cast<float*>(delta.ptr);
     const bool f32 = dt == FA_DTYPE_FLOAT32 || s.d > 256;      // vector-ALU kernels

@@ -131,6 +131,12 @@ def test_validate_fwd_error_contract():
     p.K = T4(p.K.data_ptr, p.K.sizes, [p.K.stride(0), p.K.stride(1), -128, 1], p.K.dtype)
     assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # negative stride
     p, keep = _fwd_params()
+    rows, cols = p.L.sizes
+    p.L = T2(p.L.data_ptr, [rows - 1, cols], [cols, 1], DType.kFloat32)
+    assert validate_fwd(p, 3) == E.hipErrorInvalidValue                        # L too small for B*Hq rows
+    p.L = T2(p.L.data_ptr, [rows, cols], [cols + 8, 1], DType.kFloat32)
+    assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # L rows not contiguous
+    p, keep = _fwd_params()
     p.causal_type = 1
     assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # only 0 and 3 exist
     p.causal_type = 3
