@@ -83,10 +83,11 @@ int check_act(const fa_tensor4& t, int dtype) {
   if (t.dtype != dtype) return FA_ERROR_INVALID_VALUE;
   if (t.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
   if (!aligned16(t.ptr)) return FA_ERROR_NOT_SUPPORTED;
+  // strides travel as unsigned 64-bit numbers; one above 2^63 is a negative stride
   for (int i = 0; i < 3; ++i)
-    if (t.sizes[i] > 1 && ((t.strides[i] % 8) != 0 || t.strides[i] < 0)) return FA_ERROR_NOT_SUPPORTED;
+    if (t.sizes[i] > 1 && ((t.strides[i] % 8) != 0 || (int64_t)t.strides[i] < 0)) return FA_ERROR_NOT_SUPPORTED;
   // a tile's rows are addressed with 32-bit byte offsets from the tile's first row
-  if (t.sizes[2] > 1 && t.strides[2] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
+  if (t.sizes[2] > 1 && (int64_t)t.strides[2] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
   return FA_SUCCESS;
 }
 
@@ -96,7 +97,7 @@ int check_act(const fa_tensor4& t, int dtype) {
 int check_row_stats(const fa_tensor2& t, int64_t need) {
   if (t.dtype != FA_DTYPE_FLOAT32) return FA_ERROR_INVALID_VALUE;
   if (t.sizes[1] > 1 && t.strides[1] != 1) return FA_ERROR_NOT_SUPPORTED;
-  if (t.sizes[0] > 1 && t.strides[0] != (int64_t)t.sizes[1]) return FA_ERROR_NOT_SUPPORTED;
+  if (t.sizes[0] > 1 && t.strides[0] != t.sizes[1]) return FA_ERROR_NOT_SUPPORTED;
   if ((int64_t)t.sizes[0] * (int64_t)t.sizes[1] < need) return FA_ERROR_INVALID_VALUE;
   return FA_SUCCESS;
 }
@@ -178,8 +179,8 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
         (int)B.sizes[3] != s.max_sk)
       return FA_ERROR_INVALID_VALUE;
     for (int i = 0; i < 4; ++i)
-      if (B.strides[i] < 0) return FA_ERROR_NOT_SUPPORTED;
-    if (B.strides[2] > kMaxRowStride * 8 || B.strides[3] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
+      if ((int64_t)B.strides[i] < 0) return FA_ERROR_NOT_SUPPORTED;
+    if ((int64_t)B.strides[2] > kMaxRowStride * 8 || (int64_t)B.strides[3] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
   }
   *out = s;
   return FA_SUCCESS;
@@ -262,7 +263,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
     if (!s.bias) return FA_ERROR_INVALID_VALUE;
     if (p->DB.dtype != dt) return FA_ERROR_INVALID_VALUE;
     for (int i = 0; i < 4; ++i)
-      if (p->DB.sizes[i] != p->B.sizes[i] || p->DB.strides[i] < 0) return FA_ERROR_INVALID_VALUE;
+      if (p->DB.sizes[i] != p->B.sizes[i] || (int64_t)p->DB.strides[i] < 0) return FA_ERROR_INVALID_VALUE;
   }
   int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2

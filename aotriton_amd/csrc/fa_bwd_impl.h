@@ -100,7 +100,6 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   constexpr int NT = NW * 64;
   constexpr int BN = NW * 32;
   constexpr int KS = D / 16, MB = BM / 32, DB = D / 32, TS = BM / 16;
-  constexpr int ROWB = Swz<D>::ROWB;
   constexpr int NCH = BM * D / 8;                // 16-byte chunks per tile, per tensor
   constexpr int CH = (NCH + NT - 1) / NT;        // chunks per thread, per tensor
   constexpr int LPR = D / 8;                     // lanes that share one row
@@ -466,7 +465,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       pb[E / 8][E % 8] = Tr::cvt(p1);
     };
     auto ds_el = [&](int E) {
-      const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
+      const int mb = E / 16, i = E % 16, r = i % 4;
       if (E % 4 == 0 && E + 4 < 16 * MB) d4[(E / 4 + 1) & 1] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, E / 4 + 1));
       float dpv = dp[mb][i];
       if (kDropout) dpv = keep_bit[E] ? dpv * dst.scale : 0.f;   // :239-240
@@ -492,7 +491,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int mb = 0; mb < MB; ++mb) {
         dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kVLds ? vl[k % 3] : vreg[kVLds ? 0 : k], k == 0 ? zero16 : dp[mb]);
         const int gidx = k * MB + mb;
-        if (EPG1 >= 1) {
+        if constexpr (EPG1 >= 1) {
 #pragma unroll
           for (int e = 0; e < (EPG1 >= 1 ? EPG1 : 1); ++e) {
             const int E = gidx * EPG1 + e;
@@ -543,7 +542,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
           if (t + 1 < TS) ta[(t + 1) & 1 & (kRingTa ? 0 : 1)][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, t + 1, db);
           dv[db] = Tr::mfma(ta[t & 1 & (kRingTa ? 0 : 1)][db], pb[t], dv[db]);
         }
-        if (EPG3 >= 1) {
+        if constexpr (EPG3 >= 1) {
 #pragma unroll
           for (int e = 0; e < (EPG3 >= 1 ? EPG3 : 1); ++e) {
             const int E = gidx * EPG3 + e;
@@ -672,7 +671,6 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   constexpr int NT = NW * 64;
   constexpr int BM = NW * 32;
   constexpr int KS = D / 16, MB = BN / 32, DB = D / 32, TS = BN / 16;
-  constexpr int ROWB = Swz<D>::ROWB;
   constexpr int CH = (BN * D / 8) / NT;          // 16-byte chunks per thread, per tensor
   static_assert((BN * D / 8) % NT == 0, "tile must split evenly");
 

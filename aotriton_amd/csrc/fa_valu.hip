@@ -112,7 +112,7 @@ __global__ void valu_fwd_kernel(const FwdArgs a) {
     if (a.seed_out) *a.seed_out = *a.drop.seed_ptr;
     if (a.offset_out) *a.offset_out = base;
   }
-  if (blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
+  if ((int)blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
   const bool row_ok = m < si.seqlen_q;
   const int mc = row_ok ? m : si.seqlen_q - 1;
   const int hk = h / (a.hq / a.hk);
@@ -177,7 +177,7 @@ __global__ void valu_delta_kernel(const BwdArgs a) {
   const int h = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
   const int m = blockIdx.x * kRowsPerBlock + (tid >> 3);
-  if (blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
+  if ((int)blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
   const bool row_ok = m < si.seqlen_q;
   const int mc = row_ok ? m : si.seqlen_q - 1;
   const T* op = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
@@ -195,7 +195,7 @@ __global__ void valu_dq_kernel(const BwdArgs a) {
   const int h = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
   const int m = blockIdx.x * kRowsPerBlock + (tid >> 3);
-  if (blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
+  if ((int)blockIdx.x * kRowsPerBlock >= si.seqlen_q) return;
   const bool row_ok = m < si.seqlen_q;
   const int mc = row_ok ? m : si.seqlen_q - 1;
   const int hk = h / (a.hq / a.hk);
@@ -254,7 +254,7 @@ __global__ void valu_dkdv_kernel(const BwdArgs a) {
   const int hk = blockIdx.y, z = blockIdx.z;
   const SeqInfo si = get_seq(a.seq, z);
   const int n = blockIdx.x * kRowsPerBlock + (tid >> 3);
-  if (blockIdx.x * kRowsPerBlock >= si.seqlen_k) return;
+  if ((int)blockIdx.x * kRowsPerBlock >= si.seqlen_k) return;
   const bool row_ok = n < si.seqlen_k;
   const int nc = row_ok ? n : si.seqlen_k - 1;
   const Vis vis = make_vis(a.mask, si);
