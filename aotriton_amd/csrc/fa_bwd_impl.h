@@ -83,7 +83,7 @@ struct DqSmem {     // per stage: K, V (swizzled)
 };
 
 template <int D> struct BwdTile;   // NW waves; dK/dV: BN = 32*NW keys x BM queries; dQ: BM = 32*NW queries x BN keys
-template <> struct BwdTile<64>  { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
+template <> struct BwdTile<64>  { static constexpr int NW = 4, DKDV_BM = 128, DQ_BN = 128; };
 template <> struct BwdTile<128> { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
 template <> struct BwdTile<256> { static constexpr int NW = 4, DKDV_BM = 32, DQ_BN = 32; };
 
