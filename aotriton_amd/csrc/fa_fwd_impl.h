@@ -499,7 +499,7 @@ void fwd_kernel(const FwdArgs a) {
 
 // Tile table: one entry per head dim.
 template <int D> struct FwdTile;
-template <> struct FwdTile<64>  { static constexpr int NW = 8, BN = 64; };
+template <> struct FwdTile<64>  { static constexpr int NW = 8, BN = 128; };
 template <> struct FwdTile<128> { static constexpr int NW = 8, BN = 64; };
 template <> struct FwdTile<256> { static constexpr int NW = 4, BN = 32; };
 
