@@ -323,12 +323,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         for (int e = 0; e < 8; ++e) acc += (float)och[k][e] * (float)doch[k][e];
 #pragma unroll
         for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-        if (cc0 == 0) Ds[r0 + k * RPI] = acc;
+        if (cc0 == 0) Ds[r0 + k * RPI] = kDropout ? acc : -acc;
       }
     }
     if (tid < BM) {
       Ls[tid] = l_stage * kRcpLn2;                          // bwd_inner_dk_dv.py:185-186
-      if (!kInlineDelta) Ds[tid] = d_stage;
+      // without dropout -delta is staged: it is the initial value of the dP accumulators
+      if (!kInlineDelta) Ds[tid] = kDropout ? d_stage : -d_stage;
     }
   };
 
@@ -368,6 +369,18 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Qb, row_a, k, mb);
+    if (!kDropout) {
+      // dP starts at -delta of its query rows, so dP - delta leaves the matrix pipe; with
+      // dropout the mask and the scale come between the two and the subtraction stays in ds_el
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 t4 = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 4 * mb + g));
+#pragma unroll
+          for (int r = 0; r < 4; ++r) dp[mb][4 * g + r] = t4[r];
+        }
+    }
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
       if (k + kAhead < KS) {
@@ -466,9 +479,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     };
     auto ds_el = [&](int E) {
       const int mb = E / 16, i = E % 16, r = i % 4;
+      if (!kDropout) {
+        dp[mb][i] = s[mb][i] * dp[mb][i];                         // dp already holds dP - delta
+        return;
+      }
       if (E % 4 == 0 && E + 4 < 16 * MB) d4[(E / 4 + 1) & 1] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, E / 4 + 1));
       float dpv = dp[mb][i];
-      if (kDropout) dpv = keep_bit[E] ? dpv * dst.scale : 0.f;   // :239-240
+      dpv = keep_bit[E] ? dpv * dst.scale : 0.f;                  // :239-240
       dp[mb][i] = s[mb][i] * (dpv - d4[(E / 4) & 1][r]);          // ds uses the undropped p (:242)
     };
     auto ds_pair = [&](int E) {  // E odd: ds cast to Q's dtype
@@ -489,7 +506,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       if (kVLds && k + 2 < KS) vl[(k + 2) % 3] = swz_read_row<T, D>(Vt, row_a, k + 2, wave);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kVLds ? vl[k % 3] : vreg[kVLds ? 0 : k], k == 0 ? zero16 : dp[mb]);
+        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kVLds ? vl[k % 3] : vreg[kVLds ? 0 : k],
+                          k == 0 && kDropout ? zero16 : dp[mb]);
         const int gidx = k * MB + mb;
         if constexpr (EPG1 >= 1) {
 #pragma unroll
@@ -511,7 +529,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       }
     }
     // delta of the tile's queries, first transposed dO operands
-    d4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 0));
+    if (kDropout) d4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 0));
     // Transposed operands are read ahead of their MFMAs: a whole 16-query step ahead, or,
     // where that would take too many registers (D = 256), through a ring of kRing operands.
     constexpr bool kRingTa = DB >= 8;
@@ -771,6 +789,10 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     d_row = a.delta[lo];
   }
 
+  f32x16 negd16;      // -delta of this lane's query in every element: the initial value of dP
+#pragma unroll
+  for (int i = 0; i < 16; ++i) negd16[i] = -d_row;
+
   const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
                    (int64_t)si.k_start * a.sk.s;
   const T* vbase = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
@@ -927,7 +949,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       if (kDropout && r == 0) keep[E / 4] = dropout_keep4(dst, row, n);
       float dpv = dp[mb][i];
       if (kDropout) dpv = ((keep[E / 4] >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
-      const float dsv = s[mb][i] * (dpv - d_row);
+      // without dropout the dP accumulators start at -delta, so dP - delta leaves the matrix pipe
+      const float dsv = kDropout ? s[mb][i] * (dpv - d_row) : s[mb][i] * dpv;
       dp[mb][i] = dsv;
       if (kBias && dbptr != nullptr && row_ok) {                                 // bwd_inner_dq.py:200-204
         if (tile_vec && db_vec) {
@@ -959,7 +982,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], doreg[k], k == 0 ? zero16 : dp[mb]);
+        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], doreg[k], k == 0 ? (kDropout ? zero16 : negd16) : dp[mb]);
 #pragma unroll
         for (int e = 0; e < EPG1; ++e) p_el((k * MB + mb) * EPG1 + e);
         __builtin_amdgcn_sched_barrier(0);
