@@ -313,6 +313,55 @@ def test_sampled_strides_bias_layouts_and_masks(i):
         check('db', bg.grad, rg[3], lg[3], FUDGE['db'])
 
 
+def test_concurrent_streams_and_threads_give_the_serial_results():
+    """Calls are re-entrant and ordered only by the stream they are given: three host threads,
+    each on its own stream with its own shape, repeat forward + backward; every result must
+    equal the one computed alone on the default stream, bit for bit (both backends are
+    deterministic)."""
+    import threading
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    shapes = [(2, 8, 4, 1024, 128, torch.bfloat16, True, 0), (1, 6, 6, 777, 64, torch.float16, False, 1),
+              (3, 4, 1, 300, 256, torch.bfloat16, (50, 10), 0)]
+    g = torch.Generator().manual_seed(9)
+    cases = []
+    for B, Hq, Hk, S, D, dtype, causal, be in shapes:
+        rn = lambda *sh: torch.randn(*sh, generator=g).to(dtype).to(DEV)
+        cases.append((rn(B, Hq, S, D), rn(B, Hk, S, D), rn(B, Hk, S, D), rn(B, Hq, S, D), causal, be, D))
+
+    def run(case):
+        q, k, v, do, causal, be, D = case
+        qg, kg, vg = [t.clone().requires_grad_() for t in (q, k, v)]
+        o, _, L = attention(qg, kg, vg, None, causal, D ** -0.5, 0.0,
+                            AttentionExtraArgs(return_logsumexp=True, bwd_backend=be))
+        o.backward(do)
+        return [o.detach(), L, qg.grad, kg.grad, vg.grad]
+
+    serial = [run(c) for c in cases]
+    torch.cuda.synchronize()
+    results = [None] * len(cases)
+    errors = []
+
+    def worker(i):
+        try:
+            st = torch.cuda.Stream()
+            st.wait_stream(torch.cuda.default_stream())
+            with torch.cuda.stream(st):
+                for _ in range(5):
+                    results[i] = run(cases[i])
+            st.synchronize()
+        except Exception as e:       # surfaces in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(cases))]
+    for t in threads: t.start()
+    for t in threads: t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for a, b in zip(serial, results):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+
 @pytest.mark.parametrize('causal', [1, 2])
 def test_bottom_right_and_top_left_with_sq_gt_sk(causal):
     # rows with no visible key: O = 0, LSE = +inf, gradients finite
