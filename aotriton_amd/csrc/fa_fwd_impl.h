@@ -213,6 +213,26 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     wave_hi = cmax < 0 ? -1 : (int)(cmax / BN);
   }
 
+  // A K tile needs no mask in this wave when every key of it is visible to every (valid) row of
+  // the wave: the tile ends inside the sequence, at or before the first row's right bound, and
+  // starts at or after the last row's left bound.
+  const int w_rmin = q0 + wave * 32;
+  const int w_rmax = w_rmin + 31 < si.seqlen_q ? w_rmin + 31 : si.seqlen_q - 1;
+  auto wave_sees_all = [&](int j) -> bool {
+    const int n_first = j * BN, n_last = j * BN + BN - 1;
+    bool all = n_last < si.seqlen_k;
+    if (kWindowed) all = all && n_last <= w_rmin + w.right && n_first >= w_rmax - w.left;
+    return all;
+  };
+  // visible columns of this lane's row as one range [m_lo, m_lo + m_rng] (empty: m_rng < 0)
+  int m_lo = 0, m_hi = si.seqlen_k - 1;
+  if (kWindowed) {
+    m_lo = row - w.left > 0 ? row - w.left : 0;
+    m_hi = row + w.right < m_hi ? row + w.right : m_hi;
+  }
+  const bool m_none = m_hi < m_lo;
+  const unsigned m_rng = m_none ? 0u : (unsigned)(m_hi - m_lo);
+
   f32x16 s[MB];   // S^T of the current tile
 
   auto qk = [&](int stage) {
@@ -275,13 +295,14 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
       }
     }
     if (masked) {
+      // column n of element (mb, i) is visible iff m_lo <= n <= m_hi, tested as one unsigned
+      // comparison of n - m_lo; an empty range fails every element
+      const unsigned d = m_none ? 0x40000000u : (unsigned)(j * BN + 4 * hi - m_lo);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int n = j * BN + mb * 32 + 8 * (i / 4) + 4 * hi + (i % 4);
-          bool vis = n < si.seqlen_k;
-          if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
+          const bool vis = d + (unsigned)(mb * 32 + 8 * (i / 4) + (i % 4)) <= m_rng;
           s[mb][i] = vis ? s[mb][i] : -__builtin_inff();
         }
     }
@@ -416,7 +437,8 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     if (j < br.hi) load_next_tile();
     if (j <= wave_hi) {
       qk(stage);
-      const bool masked = !br.is_full(j);
+      // per-element masks only where some row of this wave has a hidden key in the tile
+      const bool masked = !br.is_full(j) && !wave_sees_all(j);
       if (!(have_ref && sv_fast(j, stage, masked))) {
         if (have_ref) qk(stage);      // the speculative step consumed S
         sv(j, stage, masked);
