@@ -28,7 +28,7 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16/fp16 MFMA: 256 CU x 2.4 GHz x
 # HBM bytes per launch at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # runs scaled by a 256 MiB elementwise probe (summaries and commands: profiles/*.txt).
 # Counters cannot be read from inside this process, so the figures are recorded here.
-HBM_BYTES_PER_LAUNCH = {'fwd_kernel': 6.9092e8, 'bwd_dkdv_kernel': 8.1996e8, 'bwd_dq_kernel': 7.7219e8}
+HBM_BYTES_PER_LAUNCH = {'fwd_kernel': 6.9703e8, 'bwd_dkdv_kernel': 8.1939e8, 'bwd_dq_kernel': 7.7205e8}
 
 
 def cpu_baseline(B, H, S, D, causal, seed):
