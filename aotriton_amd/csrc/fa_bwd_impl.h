@@ -789,6 +789,10 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     d_row = a.delta[lo];
   }
 
+  // Without dropout (the mask and the scale come between dP and the subtraction) dP starts at
+  // -delta.  Not at D = 64: with 128-key tiles the register allocation of that kernel gets
+  // worse with the extra tuple (dQ kernel 20-50 % slower).
+  constexpr bool kFoldDelta = !kDropout && D >= 128;
   f32x16 negd16;      // -delta of this lane's query in every element: the initial value of dP
 #pragma unroll
   for (int i = 0; i < 16; ++i) negd16[i] = -d_row;
@@ -949,8 +953,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       if (kDropout && r == 0) keep[E / 4] = dropout_keep4(dst, row, n);
       float dpv = dp[mb][i];
       if (kDropout) dpv = ((keep[E / 4] >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
-      // without dropout the dP accumulators start at -delta, so dP - delta leaves the matrix pipe
-      const float dsv = kDropout ? s[mb][i] * (dpv - d_row) : s[mb][i] * dpv;
+      // where the dP accumulators start at -delta, dP - delta leaves the matrix pipe
+      const float dsv = kFoldDelta ? s[mb][i] * dpv : s[mb][i] * (dpv - d_row);
       dp[mb][i] = dsv;
       if (kBias && dbptr != nullptr && row_ok) {                                 // bwd_inner_dq.py:200-204
         if (tile_vec && db_vec) {
@@ -982,7 +986,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], doreg[k], k == 0 ? (kDropout ? zero16 : negd16) : dp[mb]);
+        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], doreg[k], k == 0 ? (kFoldDelta ? negd16 : zero16) : dp[mb]);
 #pragma unroll
         for (int e = 0; e < EPG1; ++e) p_el((k * MB + mb) * EPG1 + e);
         __builtin_amdgcn_sched_barrier(0);
