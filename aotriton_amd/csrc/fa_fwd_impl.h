@@ -213,6 +213,9 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     wave_hi = cmax < 0 ? -1 : (int)(cmax / BN);
   }
 
+  // (At D = 256 the extra lane state costs the one-wave-per-SIMD kernel 2-3 %, so it keeps the
+  // plain test on every masked tile.)
+  constexpr bool kWaveMask = D <= 128;
   // A K tile needs no mask in this wave when every key of it is visible to every (valid) row of
   // the wave: the tile ends inside the sequence, at or before the first row's right bound, and
   // starts at or after the last row's left bound.
@@ -294,7 +297,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
           }
       }
     }
-    if (masked) {
+    if (masked && kWaveMask) {
       // column n of element (mb, i) is visible iff m_lo <= n <= m_hi, tested as one unsigned
       // comparison of n - m_lo; an empty range fails every element
       const unsigned d = m_none ? 0x40000000u : (unsigned)(j * BN + 4 * hi - m_lo);
@@ -303,6 +306,16 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const bool vis = d + (unsigned)(mb * 32 + 8 * (i / 4) + (i % 4)) <= m_rng;
+          s[mb][i] = vis ? s[mb][i] : -__builtin_inff();
+        }
+    } else if (masked) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int n = j * BN + mb * 32 + 8 * (i / 4) + 4 * hi + (i % 4);
+          bool vis = n < si.seqlen_k;
+          if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
           s[mb][i] = vis ? s[mb][i] : -__builtin_inff();
         }
     }
@@ -438,7 +451,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     if (j <= wave_hi) {
       qk(stage);
       // per-element masks only where some row of this wave has a hidden key in the tile
-      const bool masked = !br.is_full(j) && !wave_sees_all(j);
+      const bool masked = !br.is_full(j) && !(kWaveMask && wave_sees_all(j));
       if (!(have_ref && sv_fast(j, stage, masked))) {
         if (have_ref) qk(stage);      // the speculative step consumed S
         sv(j, stage, masked);
