@@ -790,9 +790,9 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   }
 
   // Without dropout (the mask and the scale come between dP and the subtraction) dP starts at
-  // -delta.  Not at D = 64: with 128-key tiles the register allocation of that kernel gets
-  // worse with the extra tuple (dQ kernel 20-50 % slower).
-  constexpr bool kFoldDelta = !kDropout && D >= 128;
+  // -delta.  Not in the dQ kernel at D = 64: with 128-key tiles its register allocation gets
+  // worse with the extra tuple (20-50 % slower); the single-launch kernel at D = 64 gains.
+  constexpr bool kFoldDelta = !kDropout && (D >= 128 || kInlineDelta);
   f32x16 negd16;      // -delta of this lane's query in every element: the initial value of dP
 #pragma unroll
   for (int i = 0; i < 16; ++i) negd16[i] = -d_row;
