@@ -178,7 +178,7 @@ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
 
 struct DropoutState {
   uint32_t k0, k1;
-  uint64_t base;     // philox_offset2 + *philox_offset1 + (z*Hq + h)*max_seqlen_q*stride
+  uint64_t base;     // philox_offset2 + *philox_offset1 + int32((z*Hq + h)*max_seqlen_q*stride)
   uint32_t stride;   // cdiv(max_seqlen_k, 4)
   int32_t thr;
   float scale;       // 1/(1-p)
@@ -192,8 +192,10 @@ __device__ __forceinline__ DropoutState make_dropout(const DropoutArgs& d, int z
   if (d.offset1_ptr) base += *d.offset1_ptr;
   s.k0 = (uint32_t)seed; s.k1 = (uint32_t)(seed >> 32);
   s.stride = (uint32_t)((max_seqlen_k + 3) / 4);
-  // modules/flash/kernel/fwd_kernel.py:405-407
-  s.base = base + (uint64_t)(z * hq + h) * (uint64_t)max_seqlen_q * (uint64_t)s.stride;
+  // modules/flash/kernel/fwd_kernel.py:405-407: the per-head term is a product of int32
+  // values there, so it wraps modulo 2^32 and is sign-extended into the 64-bit base.
+  const uint32_t head_term = (uint32_t)(z * hq + h) * (uint32_t)max_seqlen_q * s.stride;
+  s.base = base + (uint64_t)(int64_t)(int32_t)head_term;
   s.thr = dropout_threshold(d.p);
   s.scale = 1.0f / (1.0f - d.p);
   return s;

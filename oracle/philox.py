@@ -5,6 +5,12 @@ Follows the reference's call chain:
   fast_philox        modules/flash/kernel/dropout.py:16-38
   threshold          modules/flash/kernel/fwd_kernel.py:195
   per-head base      modules/flash/kernel/fwd_kernel.py:405-407
+Pinned by tests/golden/dropout_mask_reference.npz: masks that the reference's own
+debug_simulate_encoded_softmax kernel (dropout_rng.py:86-126) wrote under Triton's CPU
+interpreter (tests/golden/make_dropout_fixture.py), including a case where the int32
+per-head term wraps.  The row term r * stride is computed exactly here; the reference
+forms it from int32 pieces that depend on its tile size, which differs only when
+Max_seqlen_q * cdiv(Max_seqlen_k, 4) reaches 2**31.
 The generator itself lives in a third-party dependency (Triton
 ``tl.randint4x`` / ``philox_impl``, submodule third_party/triton, not vendored):
 it is the published Philox-4x32 with 10 rounds (Salmon et al., SC'11) with
@@ -92,7 +98,12 @@ def dropout_keep_mask(batch, num_heads, max_seqlen_q, max_seqlen_k, dropout_p,
     cs = np.arange(stride, dtype=np.uint64)
     zh = (bs[:, None].astype(np.uint64) * np.uint64(num_heads) + hs[None, :].astype(np.uint64))
     with np.errstate(over='ignore'):
-        base = np.uint64(int(offset) & 0xFFFFFFFFFFFFFFFF) + zh * np.uint64(max_seqlen_q) * np.uint64(stride)
+        # The per-head term is a product of int32 values in the reference (off_zh *
+        # Max_seqlen_q * philox_offset_stride, fwd_kernel.py:405-407, dropout_rng.py:110):
+        # it wraps modulo 2**32 and is sign-extended when it meets the uint64 base.
+        head = (zh * np.uint64(max_seqlen_q) * np.uint64(stride)) & MASK32
+        head = head.astype(np.uint32).view(np.int32).astype(np.int64).view(np.uint64)
+        base = np.uint64(int(offset) & 0xFFFFFFFFFFFFFFFF) + head
         ctr = base[:, :, None, None] + rs[None, None, :, None] * np.uint64(stride) + cs[None, None, None, :]
     words = philox_words(seed, ctr)                       # [b,h,r,stride,4]
     words = words.reshape(len(bs), len(hs), len(rs), stride * 4)[..., :max_seqlen_k]

@@ -79,3 +79,26 @@ def check(name, out, ref_hp, ref_lp, fudge, mask=None):
             f.write(f"{os.environ.get('PYTEST_CURRENT_TEST', '?')}\t{name}\t{err:.4e}\t{ref_err:.4e}\n")
     assert err <= thr, f'{name}: max|out-ref|={err:.3e} > {thr:.3e} (ref_lp err {ref_err:.3e}, fudge {fudge})'
     return err, thr
+
+
+def reference_dropout_fixture():
+    """Masks written by the reference's own debug_simulate_encoded_softmax kernel under
+    Triton's CPU interpreter (tests/golden/make_dropout_fixture.py).  Yields dicts with
+    B, H, Sq (rows stored), max_sq (the Max_seqlen_q the kernel was given), Sk, p, seed,
+    off1, off2 and keep[B, H, Sq, Sk] (bool)."""
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'dropout_mask_reference.npz'))
+    out = []
+    i = 0
+    while f'case{i}_keep' in z:
+        B, H, Sq, Sk = (int(x) for x in z[f'case{i}_params'])
+        seed, off1, off2 = (int(x) for x in z[f'case{i}_rng'])
+        keep = np.unpackbits(z[f'case{i}_keep'])[:B * H * Sq * Sk].reshape(B, H, Sq, Sk).astype(bool)
+        out.append(dict(B=B, H=H, Sq=Sq, max_sq=Sq, Sk=Sk, p=float(z[f'case{i}_p'][0]), seed=seed, off1=off1,
+                        off2=off2, keep=keep))
+        i += 1
+    B, H, rows, max_sq, Sk = (int(x) for x in z['wrap_params'])
+    seed, off1, off2 = (int(x) for x in z['wrap_rng'])
+    keep = np.unpackbits(z['wrap_keep'])[:B * H * rows * Sk].reshape(B, H, rows, Sk).astype(bool)
+    out.append(dict(B=B, H=H, Sq=rows, max_sq=max_sq, Sk=Sk, p=float(z['wrap_p'][0]), seed=seed, off1=off1,
+                    off2=off2, keep=keep))
+    return out

@@ -233,6 +233,50 @@ def test_encoded_softmax_is_bit_exact(dtype, shape, p, state):
     assert np.array_equal((r >= 0).cpu().numpy(), keep)
 
 
+def test_mask_equals_the_reference_kernels_mask():
+    """debug_simulate_encoded_softmax and the forward's own encoded_softmax against the masks
+    that the reference's kernel wrote (tests/golden/dropout_mask_reference.npz, see
+    tests/golden/make_dropout_fixture.py)."""
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from _util import reference_dropout_fixture
+    for c in reference_dropout_fixture():
+        if c['max_sq'] != c['Sq']:
+            continue   # the int32-wrap case needs 2**27 rows: covered at full size below
+        B, H, Sq, Sk = c['B'], c['H'], c['Sq'], c['Sk']
+        sk8 = (Sk + 7) // 8 * 8
+        for dtype in (torch.float16, torch.bfloat16, torch.float32):
+            r = torch.zeros(B, H, Sq, sk8, dtype=dtype, device=DEV)[..., :Sk]
+            assert flash.debug_simulate_encoded_softmax(r, c['p'], _u64(c['seed']), _u64(c['off1']), c['off2']) == 0
+            assert np.array_equal((r >= 0).cpu().numpy(), c['keep'])
+        # the mask the forward kernel applies (returned through encoded_softmax)
+        q, k, v, _, _ = make_inputs(B, H, H, Sq, Sk, 64, torch.float16, DEV, seed=3)
+        ext = AttentionExtraArgs(return_encoded_softmax=True, philox_seed=c['seed'], philox_offset1=c['off1'],
+                                 philox_offset2=c['off2'])
+        _, enc, _ = attention(q, k, v, None, False, 0.125, c['p'], ext)
+        assert np.array_equal((enc >= 0).cpu().numpy(), c['keep'])
+
+
+def test_per_head_counter_term_wraps_in_int32():
+    """B1 H2 Sq 2^20 Sk 8192: head 1's term (1 * 2^20 * 2048 = 2^31) wraps to -2^31 as in the
+    reference (fwd_kernel.py:405-407; pinned on the CPU by the fixture's wrapping case)."""
+    from aotriton_amd import flash
+    from oracle import philox
+    H, Sq, Sk = 2, 1 << 20, 8192
+    r = torch.empty(1, H, Sq, Sk, dtype=torch.float16, device=DEV)
+    off2 = 1 << 40
+    assert flash.debug_simulate_encoded_softmax(r, 0.5, _u64(0x1234), _u64(5), off2) == 0
+    for h in range(H):
+        for m in (0, 1, 4097, Sq - 1):
+            exp = philox.dropout_keep_mask(1, H, Sq, Sk, 0.5, 0x1234, 5 + off2, rows=(m, m + 1), h_sel=[h])[0, 0, 0]
+            assert np.array_equal((r[0, h, m] >= 0).cpu().numpy(), exp), (h, m)
+    # what exact 64-bit arithmetic would have given for head 1 is a different row
+    unwrapped = philox.dropout_keep_mask(1, 1, 1, Sk, 0.5, 0x1234, 5 + off2 + (1 << 31))[0, 0, 0]
+    assert not np.array_equal((r[0, 1, 0] >= 0).cpu().numpy(), unwrapped)
+    del r
+    torch.cuda.empty_cache()
+
+
 def test_config5_mask_first_words_and_popcount():
     """BASELINE config 5 mask (seed 0x1234, offset 0, p=0.1, 8192x8192) on sampled
     (b, h) slices: bit-exact rows against the oracle and a keep-rate check."""

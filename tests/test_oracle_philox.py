@@ -36,6 +36,25 @@ def test_threshold_fp32():
     assert philox.idropout_p(0.1) != -1717986918
 
 
+def test_mask_equals_the_reference_kernels_mask():
+    """The oracle's whole-tensor mask against what the reference's own
+    debug_simulate_encoded_softmax kernel wrote (modules/flash/kernel/dropout_rng.py:86-126,
+    run under Triton's CPU interpreter by tests/golden/make_dropout_fixture.py): several batch
+    elements and heads, more than one 64-row tile, key counts off the multiples of 4 and 32,
+    a seed above 2**32, offset1 and offset2 both non-zero, a counter that carries into its
+    high word, and a per-head term that wraps in int32."""
+    from tests._util import reference_dropout_fixture
+    cases = reference_dropout_fixture()
+    assert len(cases) == 5
+    for c in cases:
+        m = philox.dropout_keep_mask(c['B'], c['H'], c['max_sq'], c['Sk'], c['p'], c['seed'],
+                                     c['off1'] + c['off2'], rows=(0, c['Sq']))
+        assert np.array_equal(m, c['keep']), (c['B'], c['H'], c['Sq'], c['Sk'])
+    # the wrapping case really wraps: exact 64-bit arithmetic gives another mask for heads 1, 2
+    c = cases[-1]
+    assert c['H'] * c['max_sq'] * ((c['Sk'] + 3) // 4) >= 2 ** 31
+
+
 def test_mask_matches_per_element_closed_form():
     B, H, Sq, Sk, p, seed, off = 2, 3, 5, 10, 0.1, 0x1234, 7
     mask = philox.dropout_keep_mask(B, H, Sq, Sk, p, seed, off)
