@@ -98,6 +98,7 @@ SYMBOLS = {
     'fa_check_gpu': (ctypes.c_int, [ctypes.c_void_p]),
     'fa_attn_fwd': (ctypes.c_int, [P(fa_fwd_params), ctypes.c_int32, ctypes.c_void_p, P(fa_options)]),
     'fa_attn_bwd': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p, P(fa_options)]),
+    'fa_attn_bwd_noalloc': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p]),
     'fa_attn_bwd_kernel': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32]),
     'fa_debug_simulate_encoded_softmax': (ctypes.c_int, [P(fa_tensor4), ctypes.c_float, P(fa_tensor0),
                                                          P(fa_tensor0), ctypes.c_uint64, ctypes.c_void_p]),

@@ -70,6 +70,35 @@ const DeviceInfo* device_of_stream(hipStream_t stream) {
   return &d;
 }
 
+int device_index(const DeviceInfo* d) { return (int)(d - g_devices); }
+
+// Delta buffer of fa_attn_bwd_noalloc: device memory that belongs to the library, one copy
+// per GPU the library runs on, held until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress; the address the kernels get is looked up once
+// per device (with that device current) and kept in g_scratch_ptr.
+constexpr int64_t kScratchFloats = FA_NOALLOC_MAX_ROWS;
+__device__ __align__(256) static float scratch[kScratchFloats];
+float* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+hipError_t scratch_of_device(int dev, float** out) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    int cur = -1;
+    hipError_t e = hipGetDevice(&cur);
+    if (e != hipSuccess) return e;
+    if (cur != dev && (e = hipSetDevice(dev)) != hipSuccess) return e;
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (cur != dev) (void)hipSetDevice(cur);
+    if (e != hipSuccess) return e;
+    if (ptr == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
+}
+
 bool is_16bit(int dt) { return dt == FA_DTYPE_FLOAT16 || dt == FA_DTYPE_BFLOAT16; }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -499,11 +528,45 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
 
 // kernel_slot < 0: the whole backward of the chosen backend; otherwise only that
 // kernel (0 delta, 1 dK/dV, 2 dQ, 3 fused).
-static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
-                         const fa_options* options, int kernel_slot) {
+// own_delta: the split backend with delta in the library's own per-device array (params->D is
+// not looked at).
+static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void* hip_stream,
+                         const fa_options* options, int kernel_slot, bool own_delta = false) {
   Shape s{};
   int backend = 0;
   fa_options forced{};
+  const fa_bwd_params* p = p_in;
+  fa_bwd_params with_delta;
+  if (own_delta) {
+    if (p_in == nullptr) return FA_ERROR_INVALID_VALUE;
+    if (params_version != FA_BWD_PARAMS_VERSION) return FA_ERROR_INVALID_SYMBOL;
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    const DeviceInfo* dv = device_of_stream(st);
+    if (dv == nullptr || !dv->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+    float* ptr = nullptr;
+    hipError_t se = scratch_of_device(device_index(dv), &ptr);
+    if (se != hipSuccess) return (int)se;
+    with_delta = *p_in;
+    with_delta.D = fa_lazy_tensor2{};
+    with_delta.D.eager.ptr = ptr;
+    // sized for the check of the tensors below; the limit of the array is tested right after
+    with_delta.D.eager.sizes[0] = 1; with_delta.D.eager.sizes[1] = (uint64_t)1 << 60;
+    with_delta.D.eager.strides[0] = (uint64_t)1 << 60; with_delta.D.eager.strides[1] = 1;
+    with_delta.D.eager.dtype = FA_DTYPE_FLOAT32;
+    p = &with_delta;
+    forced.force_backend_index = 0;
+    forced.deterministic = 0;
+    options = &forced;
+    Shape probe{};
+    const int pe = validate_bwd(p, params_version, options, &probe, nullptr);
+    if (pe != FA_SUCCESS) return pe;
+    // one delta value per (batch element or token, query head, query row)
+    if (probe.row_stats > kScratchFloats) {
+      FA_LOG(1, "attn_bwd_noalloc: %lld delta values needed, the library's array holds %lld",
+             (long long)probe.row_stats, (long long)kScratchFloats);
+      return FA_ERROR_OUT_OF_MEMORY;
+    }
+  }
   if (kernel_slot >= 0) {
     forced.force_backend_index = kernel_slot == 3 ? 1 : 0;
     forced.deterministic = 0;
@@ -574,6 +637,10 @@ static int attn_bwd_impl(const fa_bwd_params* p, int32_t params_version, void* h
 int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
                 const fa_options* options) {
   return attn_bwd_impl(p, params_version, hip_stream, options, -1);
+}
+
+int fa_attn_bwd_noalloc(const fa_bwd_params* p, int32_t params_version, void* hip_stream) {
+  return attn_bwd_impl(p, params_version, hip_stream, nullptr, -1, true);
 }
 
 int fa_attn_bwd_kernel(const fa_bwd_params* p, int32_t params_version, void* hip_stream,

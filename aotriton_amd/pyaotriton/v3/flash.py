@@ -134,6 +134,13 @@ def attn_bwd(params, params_version, stream, options=None):
     return hipError_t(lib.fa_attn_bwd(ctypes.byref(c), int(params_version), stream.native() or None, optp))
 
 
+def attn_bwd_noalloc(params, params_version, stream):
+    """Split backward with delta in the library's own device array: allocates nothing, ignores
+    params.D; at most FA_NOALLOC_MAX_ROWS delta values (hipErrorOutOfMemory beyond)."""
+    c = params.to_c()
+    return hipError_t(lib.fa_attn_bwd_noalloc(ctypes.byref(c), int(params_version), stream.native() or None))
+
+
 def attn_bwd_kernel(params, params_version, stream, kernel_slot):
     """Launch one backward kernel only (0 delta, 1 dK/dV, 2 dQ, 3 fused)."""
     c = params.to_c()

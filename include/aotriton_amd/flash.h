@@ -52,6 +52,7 @@ enum fa_dtype {
 enum fa_error {
   FA_SUCCESS = 0,
   FA_ERROR_INVALID_VALUE = 1,             /* null / inconsistent tensor views            */
+  FA_ERROR_OUT_OF_MEMORY = 2,             /* fa_attn_bwd_noalloc: more rows than its array holds */
   FA_ERROR_INVALID_SYMBOL = 13,           /* params_version mismatch                     */
   FA_ERROR_NO_BINARY_FOR_GPU = 209,       /* device is not gfx950                        */
   FA_ERROR_PEER_ACCESS_UNSUPPORTED = 217, /* a forced backend cannot take this input     */
@@ -215,6 +216,18 @@ FA_API int fa_attn_fwd(const fa_fwd_params* params, int32_t params_version,
  * modules/flash/csrc/attn_bwd.cc:55-160. */
 FA_API int fa_attn_bwd(const fa_bwd_params* params, int32_t params_version,
                        void* hip_stream, const fa_options* options);
+
+/* The split backward for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same inputs, outputs and
+ * results as fa_attn_bwd with backend 0, but delta lives in a device array that belongs to
+ * the library (FA_NOALLOC_MAX_ROWS floats = 16 MiB per GPU the library runs on, held until the
+ * process ends); params->D is ignored and nothing is allocated or freed.  It has no
+ * counterpart in the reference.  Needs batch * Hq * max_seqlen_q (packed sequences: Hq * tokens)
+ * <= FA_NOALLOC_MAX_ROWS, else FA_ERROR_OUT_OF_MEMORY before any launch.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (two streams, two threads) race. */
+#define FA_NOALLOC_MAX_ROWS (4 * 1024 * 1024)
+FA_API int fa_attn_bwd_noalloc(const fa_bwd_params* params, int32_t params_version,
+                               void* hip_stream);
 
 /* One kernel of the backward only: kernel_slot 0 = delta (bwd_preprocess), 1 = dK/dV,
  * 2 = dQ, 3 = fused.  Slots 0-2 need an eager delta buffer in params->D.  Stands in
