@@ -209,7 +209,8 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
       return FA_ERROR_INVALID_VALUE;
     for (int i = 0; i < 4; ++i)
       if ((int64_t)B.strides[i] < 0) return FA_ERROR_NOT_SUPPORTED;
-    if ((int64_t)B.strides[2] > kMaxRowStride * 8 || (int64_t)B.strides[3] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
+    // bias rows of a tile are addressed with 32-bit byte offsets, like the activations'
+    if ((int64_t)B.strides[2] > kMaxRowStride || (int64_t)B.strides[3] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
   }
   *out = s;
   return FA_SUCCESS;

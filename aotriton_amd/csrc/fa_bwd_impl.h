@@ -1166,12 +1166,12 @@ inline int persistent_workers(const BwdArgs& a) {
   return w > a.items_per_xcd ? a.items_per_xcd : w;
 }
 
-template <typename K>
-hipError_t launch_with_lds(K kern, dim3 grid, int nthreads, int smem, hipStream_t stream, const BwdArgs& a) {
+template <auto kern>
+hipError_t launch_with_lds(dim3 grid, int nthreads, int smem, hipStream_t stream, const BwdArgs& a) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;   // an empty tensor: nothing to write
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static std::atomic<uint64_t> lds_set{0};
+    hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern), smem, lds_set);
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(nthreads), smem, stream, a);
@@ -1209,7 +1209,7 @@ hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dro
   a.zh_group = 2;
   a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles;
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
-#define FA_CALL(W, B, P) launch_with_lds(bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>, grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
+#define FA_CALL(W, B, P) launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>>(grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
@@ -1224,7 +1224,7 @@ hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropo
   a.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
   a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_m_tiles;
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
-#define FA_CALL(W, B, P) launch_with_lds(bwd_dq_kernel<T, D, NW, BN, W, B, P, kPad>, grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
+#define FA_CALL(W, B, P) launch_with_lds<bwd_dq_kernel<T, D, NW, BN, W, B, P, kPad>>(grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
@@ -1241,7 +1241,7 @@ hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dr
   a.zh_group = 2;
   const int items = a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk);
   dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * items));
-#define FA_CALL(W, B, P) launch_with_lds(bwd_fused_kernel<T, D, NW, BM, BN, W, B, P, kPad>, grid, NW * 64, smem, stream, a)
+#define FA_CALL(W, B, P) launch_with_lds<bwd_fused_kernel<T, D, NW, BM, BN, W, B, P, kPad>>(grid, NW * 64, smem, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }

@@ -14,10 +14,26 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "fa_args.h"
 #include "fa_intervals.h"
 
 namespace fa {
+
+// Kernels with more than 64 KB of LDS need hipFuncAttributeMaxDynamicSharedMemorySize, which is a
+// property of the function on one device: set on the first launch per (kernel, device), `done`
+// being the kernel's own bit mask of devices.
+inline hipError_t allow_large_lds(const void* kern, int smem, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 typedef __bf16 bf16_t;
 typedef _Float16 f16_t;

@@ -545,8 +545,8 @@ hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
   constexpr int smem = FwdSmem<D, BN, NW>::BYTES;
   if (grid.x == 0) return hipSuccess;      // no batch, no head or no query row: nothing to write
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static std::atomic<uint64_t> lds_set{0};
+    hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern), smem, lds_set);
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, grid, dim3(NW * 64), smem, stream, a);

@@ -32,66 +32,53 @@ class WindowValue:
 IVARLEN_TYPE = {'compact': 1, 'padded': 2, 'strided': 3}
 
 
+_TL = WindowValue.TOP_LEFT_ALIGNED
+_BR = WindowValue.BOTTOM_RIGHT_ALIGNED
+# what the v3 params carry for each way of saying "causal": (causal_type, window_left, window_right)
+_CAUSAL_OF_ENUM = {
+    CausalType.NONE: (CausalType.NONE, 0, 0),
+    CausalType.TOP_LEFT: (CausalType.WINDOWED, _TL, _TL),
+    CausalType.BOTTOM_RIGHT: (CausalType.WINDOWED, _BR, _BR),
+}
+
+
 def translate_causal(causal, v3_api=True):
-    """aotriton_flash.py:38-63: bool / (left, right) / CausalType -> (type, left, right)."""
-    window_left, window_right = 0, 0
+    """(causal_type, window_left, window_right) of the v3 params for a bool, a (left, right)
+    window or a CausalType; same mapping as aotriton_flash.py:38-63.  Only the bool form exists
+    in the v2 API."""
+    if isinstance(causal, bool):
+        return _CAUSAL_OF_ENUM[CausalType.TOP_LEFT if causal else CausalType.NONE]
+    assert v3_api, 'windows and alignment enums need the v3 params'
     if isinstance(causal, tuple):
-        assert v3_api
-        window_left, window_right = causal
-        causal_type = CausalType.WINDOWED
-    elif isinstance(causal, bool):
-        causal_type = CausalType.WINDOWED if causal else CausalType.NONE
-        if causal:
-            window_left = WindowValue.TOP_LEFT_ALIGNED
-            window_right = WindowValue.TOP_LEFT_ALIGNED
-    else:
-        assert causal in [CausalType.NONE, CausalType.TOP_LEFT, CausalType.BOTTOM_RIGHT]
-        assert v3_api
-        if causal == CausalType.TOP_LEFT:
-            causal_type = CausalType.WINDOWED
-            window_left = window_right = WindowValue.TOP_LEFT_ALIGNED
-        elif causal == CausalType.BOTTOM_RIGHT:
-            causal_type = CausalType.WINDOWED
-            window_left = window_right = WindowValue.BOTTOM_RIGHT_ALIGNED
-        else:
-            causal_type = causal
-    return causal_type, window_left, window_right
-
-
-_DTYPES = {}
+        left, right = causal
+        return CausalType.WINDOWED, left, right
+    return _CAUSAL_OF_ENUM[causal]
 
 
 def cast_dtype(dtype):
-    """aotriton_flash.py:83-91."""
-    r = _DTYPES.get(dtype)
-    if r is None:
-        r = _DTYPES[dtype] = _cast_dtype(dtype)
-    return r
-
-
-def _cast_dtype(dtype):
+    """torch dtype -> DType of the bindings (aotriton_flash.py:83-91): k<Float|BFloat|Int|UInt><bits>."""
+    import torch
+    family = ('BFloat' if dtype == torch.bfloat16 else 'Float') if dtype.is_floating_point else \
+             ('Int' if dtype.is_signed else 'UInt')
     assert not dtype.is_complex
-    bits = dtype.itemsize * 8
-    if dtype.is_floating_point:
-        maintype = 'Float' if 'bfloat' not in str(dtype) else 'BFloat'
-    else:
-        maintype = 'Int' if 'uint' not in str(dtype) else 'UInt'
-    return getattr(DType, f'k{maintype}{bits}')
+    return getattr(DType, f'k{family}{8 * dtype.itemsize}')
+
+
+_VIEW_OF_RANK = {1: T1, 2: T2, 4: T4}
 
 
 def mk_aotensor(q, if_empty_then_like=None):
-    """aotriton_flash.py:93-114: rank -> T0/T1/T2/T4; 1-D tensors with 0 or 1
-    elements become device scalars; None becomes a null view typed like
-    ``if_empty_then_like``; the last stride must be 1."""
-    rank = len(q.shape) if q is not None else len(if_empty_then_like.shape)
-    if q is not None and len(q.shape) == 1 and q.numel() in [0, 1]:
-        return T0(q.data_ptr(), cast_dtype(q.dtype))
-    klass = {1: T1, 2: T2, 4: T4}.get(rank)
-    assert klass is not None, f'Unsupported tensor rank {rank}'
+    """Tensor -> view of the bindings (aotriton_flash.py:93-114).  A 1-D tensor with at most one
+    element is a device scalar (T0); None is a null view with the rank and dtype of
+    ``if_empty_then_like``; other tensors need rank 1, 2 or 4 and a unit last stride."""
     if q is None:
-        return klass(0, [0] * rank, [0] * rank, cast_dtype(if_empty_then_like.dtype))
+        like = if_empty_then_like
+        return _VIEW_OF_RANK[like.dim()](0, [0] * like.dim(), [0] * like.dim(), cast_dtype(like.dtype))
+    if q.dim() == 1 and q.numel() <= 1:
+        return T0(q.data_ptr(), cast_dtype(q.dtype))
+    assert q.dim() in _VIEW_OF_RANK, f'Unsupported tensor rank {q.dim()}'
     assert q.stride(-1) == 1, 'the last stride of tensors must be 1'
-    return klass(q.data_ptr(), tuple(q.size()), q.stride(), cast_dtype(q.dtype))
+    return _VIEW_OF_RANK[q.dim()](q.data_ptr(), tuple(q.size()), q.stride(), cast_dtype(q.dtype))
 
 
 def _stream():

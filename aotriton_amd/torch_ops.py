@@ -34,10 +34,17 @@ def _causal_arg(causal_type, window_left, window_right):
     return (window_left, window_right) if causal_type != 0 else False
 
 
-@torch.library.custom_op('aotriton_amd::philox_state', mutates_args=(), device_types='cuda')
+@torch.library.custom_op('aotriton_amd::philox_state', mutates_args=(), device_types='cuda',
+                         tags=(torch.Tag.nondeterministic_seeded,))
 def philox_state(like: Tensor, increment: int) -> Tuple[Tensor, Tensor]:
     """Seed and offset (uint64[1] tensors on like's device) of the device's default generator;
-    the generator's offset moves on by `increment` counters (rounded up to a multiple of 4)."""
+    the generator's offset moves on by `increment` counters (rounded up to a multiple of 4).
+
+    The op reads and advances host-side generator state, so it is tagged as a seeded random op:
+    graph passes must not merge two calls or recompute one.  Under CUDA/HIP graph capture the
+    host read happens once, at capture: every replay would reuse the captured seed and offset.
+    Callers that replay graphs pass their own seed / offset tensors to flash_attention_forward
+    and update them on the device between replays."""
     gen = torch.cuda.default_generators[like.device.index]
     seed, offset = gen.initial_seed(), gen.get_offset()
     gen.set_offset(offset + (increment + 3) // 4 * 4)

@@ -131,6 +131,12 @@ def test_validate_fwd_error_contract():
     p.K = T4(p.K.data_ptr, p.K.sizes, [p.K.stride(0), p.K.stride(1), -128, 1], p.K.dtype)
     assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # negative stride
     p, keep = _fwd_params()
+    bias = torch.zeros(2, 4, 64, 80, dtype=torch.bfloat16)
+    p.B = flash_mk(bias)
+    assert validate_fwd(p, 3) == E.hipSuccess
+    p.B = T4(p.B.data_ptr, p.B.sizes, [p.B.stride(0), p.B.stride(1), (1 << 21) + 8, 1], p.B.dtype)
+    assert validate_fwd(p, 3) == E.hipErrorNotSupported                        # bias row stride beyond 32-bit tile offsets
+    p, keep = _fwd_params()
     rows, cols = p.L.sizes
     p.L = T2(p.L.data_ptr, [rows - 1, cols], [cols, 1], DType.kFloat32)
     assert validate_fwd(p, 3) == E.hipErrorInvalidValue                        # L too small for B*Hq rows
