@@ -112,6 +112,9 @@ SYMBOLS = {
     'fa_version': (ctypes.c_char_p, []),
     'fa_get_arch': (ctypes.c_int, [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int32]),
     'fa_get_multiprocessor_count': (ctypes.c_int, [ctypes.c_void_p]),
+    'fa_get_clock_rate_khz': (ctypes.c_int, [ctypes.c_void_p]),
+    'fa_probe_mfma_rate': (ctypes.c_int, [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
+                                          ctypes.c_void_p, ctypes.c_void_p]),
     'fa_hip_get_last_error': (ctypes.c_int, []),
     'fa_hip_device_synchronize': (ctypes.c_int, []),
 }

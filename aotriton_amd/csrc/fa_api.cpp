@@ -40,6 +40,7 @@ struct DeviceInfo {
   std::atomic<int> state{0};   // 0 unknown, 1 filled
   bool is_gfx950 = false;
   int num_cu = 0;
+  int clock_khz = 0;
   char arch[32] = {0};
 };
 DeviceInfo g_devices[kMaxDevices];
@@ -66,6 +67,7 @@ const DeviceInfo* device_of_stream(hipStream_t stream) {
   d.arch[n] = 0;
   d.is_gfx950 = std::strcmp(d.arch, "gfx950") == 0;
   d.num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 40;
+  d.clock_khz = prop.clockRate;
   d.state.store(1, std::memory_order_release);
   return &d;
 }
@@ -350,6 +352,21 @@ int fa_get_arch(void* hip_stream, char* buf, int32_t buflen) {
 int fa_get_multiprocessor_count(void* hip_stream) {
   const DeviceInfo* d = device_of_stream(static_cast<hipStream_t>(hip_stream));
   return d ? d->num_cu : 40;   // v3src/util.cc:95-112 falls back to 40
+}
+
+int fa_get_clock_rate_khz(void* hip_stream) {
+  const DeviceInfo* d = device_of_stream(static_cast<hipStream_t>(hip_stream));
+  return d ? d->clock_khz : 0;
+}
+
+int fa_probe_mfma_rate(int32_t random_operands, int32_t num_workgroups, int32_t iters, float* out,
+                       uint64_t* clocks, void* hip_stream) {
+  if (out == nullptr || clocks == nullptr || num_workgroups <= 0 || iters <= 0) return FA_ERROR_INVALID_VALUE;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const DeviceInfo* d = device_of_stream(stream);
+  if (d == nullptr || !d->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+  return (int)fa::run_mfma_rate(random_operands != 0, num_workgroups, iters, out,
+                                reinterpret_cast<unsigned long long*>(clocks), stream);
 }
 
 int fa_hip_get_last_error(void) { return (int)hipGetLastError(); }

@@ -20,6 +20,8 @@ hipError_t run_fwd_d256_padded(int dtype, const FwdArgs& a, bool windowed, bool 
 TileShape fwd_tile_shape(int head_dim);
 
 hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s);
+// register-only MFMA loop: the rate the matrix pipe sustains (benchmark aid)
+hipError_t run_mfma_rate(bool random_operands, int grid, int iters, float* out, unsigned long long* clk, hipStream_t s);
 
 // backward: kernel_slot 0 = preprocess (delta), 1 = dK/dV, 2 = dQ, 3 = fused
 hipError_t run_bwd_preprocess(int dtype, int head_dim, const BwdArgs& a, hipStream_t s);

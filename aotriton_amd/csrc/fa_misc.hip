@@ -42,6 +42,48 @@ hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s) {
   return hipGetLastError();
 }
 
+// Register-only loop of v_mfma_f32_32x32x16_bf16 (4 independent accumulators per wave, 8 waves
+// per CU): what the matrix pipe sustains on this machine, on constant operands or on operands
+// with random mantissas (the clock under load depends on the data).  clk[0] = shader cycles,
+// clk[1] = 100 MHz reference ticks of workgroup 0.
+template <bool kRandom>
+__global__ __launch_bounds__(256) void mfma_rate_kernel(float* out, int iters, unsigned long long* clk) {
+  using op_t = Traits<bf16_t>::op_t;
+  op_t a[8], b[8];
+  unsigned s = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+  for (int j = 0; j < 8; ++j)
+    for (int i = 0; i < 8; ++i) {
+      s = s * 1664525u + 1013904223u;
+      const float fa = kRandom ? ((int)(s >> 8) % 2001 - 1000) * 1e-3f : 1.0f;
+      s = s * 1664525u + 1013904223u;
+      const float fb = kRandom ? ((int)(s >> 8) % 2001 - 1000) * 1e-3f : 0.5f;
+      a[j][i] = (bf16_t)fa; b[j][i] = (bf16_t)fb;
+    }
+  f32x16 acc[4];
+  for (int n = 0; n < 4; ++n)
+    for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int n = 0; n < 4; ++n) acc[n] = Traits<bf16_t>::mfma(a[j], b[(j + n) & 7], acc[n]);
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+  float r = 0.f;
+  for (int n = 0; n < 4; ++n)
+    for (int i = 0; i < 16; ++i) r += acc[n][i];
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (blockIdx.x == 0 && threadIdx.x == 0) { clk[0] = t1 - t0; clk[1] = r1 - r0; }
+}
+
+// out: grid * 256 floats, clk: 2 x u64.  FLOP of one launch = grid * 4 waves * iters * 32 MFMAs * 32768.
+hipError_t run_mfma_rate(bool random_operands, int grid, int iters, float* out, unsigned long long* clk, hipStream_t s) {
+  if (random_operands) hipLaunchKernelGGL(mfma_rate_kernel<true>, dim3(grid), dim3(256), 0, s, out, iters, clk);
+  else hipLaunchKernelGGL(mfma_rate_kernel<false>, dim3(grid), dim3(256), 0, s, out, iters, clk);
+  return hipGetLastError();
+}
+
 TileShape fwd_tile_shape(int head_dim);
 
 }  // namespace fa

@@ -7,16 +7,22 @@ from a seed, sm_scale = 1/sqrt(128), inputs resident in HBM.  FLOP conventions
 are the reference's (modules/flash/tests/performance_forward.py:108-113):
 forward 4*B*H*S^2*D*0.5 (causal), backward 2.5x forward.
 
-Prints ONE JSON line.  `value` is the whole step's TFLOPS; the forward and both
-backward variants are reported separately next to it, each also as a fraction of
-the dense bf16 MFMA peak.  `roofline` describes the kernel that takes the largest
-share of the step; `cpu_baseline` is PyTorch's math SDPA (the reference's own test
-oracle) on the host CPU on a bounded sample of the same workload.
+Prints ONE JSON line.  `value` is the whole step's TFLOPS over K back-to-back steps.
+The forward, both backward variants and the single kernels are timed one launch at a
+time the way the reference times kernels (python/tune/gpu_utils.py:293-370): a buffer
+larger than the last-level cache is zeroed before every launch, warm-up >= 25 ms,
+>= 100 ms of timed launches, HIP events on the launch stream, median with the 20th and
+80th percentile.  `roofline` describes the kernel that takes the largest share of the
+step; `cpu_baseline` is PyTorch's math SDPA (the reference's own test oracle) on the host
+CPU on a bounded sample of the same workload.  `c4` and `c5` time BASELINE.json's
+configurations 4 (GQA, 16 packed sequences) and 5 (D=256, window + bias + dropout) at
+full size; they are extra keys, `value` stays the headline.
 """
 import argparse
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -24,11 +30,20 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16/fp16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+FLUSH_BYTES = 512 << 20        # zeroed before each timed launch: above the 256 MB last-level cache
 
-# HBM bytes per launch at the headline shape, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# runs scaled by a 256 MiB elementwise probe (summaries and commands: profiles/*.txt).
-# Counters cannot be read from inside this process, so the figures are recorded here.
-HBM_BYTES_PER_LAUNCH = {'fwd_kernel': 6.9703e8, 'bwd_dkdv_kernel': 8.1939e8, 'bwd_dq_kernel': 7.7205e8}
+
+def hbm_bytes_from_profile(kernel):
+    """HBM bytes per launch of `kernel` at the headline shape: the 'total ... B' figure of the
+    committed rocprofv3 summary of that kernel (FETCH_SIZE / WRITE_SIZE runs, scaled by a
+    256 MiB elementwise probe).  Counters cannot be read from inside this process."""
+    names = {'fwd_kernel': 'attn_fwd', 'bwd_dkdv_kernel': 'bwd_dkdv', 'bwd_dq_kernel': 'bwd_dq'}
+    path = os.path.join(ROOT, 'profiles', f'{names.get(kernel, kernel)}_b4_h32_s4096_d128_bf16_causal.txt')
+    try:
+        m = re.search(r'total ([0-9.e+]+) B', open(path).read())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def cpu_baseline(B, H, S, D, causal, seed):
@@ -36,7 +51,7 @@ def cpu_baseline(B, H, S, D, causal, seed):
     batch element (fp32, the precision the reference's oracle runs at)."""
     import torch
     from oracle import fa_ref
-    threads = min(os.cpu_count() or 1, 16)
+    threads = min(os.cpu_count() or 1, 16)        # a one-GPU box gives a job 16 cores
     torch.set_num_threads(threads)
     h_s = 8
     g = torch.Generator().manual_seed(seed)
@@ -59,6 +74,7 @@ def cpu_baseline(B, H, S, D, causal, seed):
     flops = 3.5 * 4.0 * 1 * h_s * S * S * D * (0.5 if causal else 1.0)
     return {
         'value': flops / dt / 1e12, 'unit': 'TFLOPS', 'cores': threads, 'kind': 'port',
+        'os_cpu_count': os.cpu_count(), 'torch_num_threads': torch.get_num_threads(),
         'sample': f'fwd+bwd of {h_s} heads of one batch element (fp32, S={S}, D={D}, causal={causal}), '
                   f'{reps} reps, {dt:.2f} s each; same FLOP formula as the GPU rows',
     }
@@ -70,22 +86,80 @@ def main():
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu', action='store_true', help='skip the host-CPU baseline leg')
+    ap.add_argument('--no-extra', action='store_true', help='skip configurations 4 and 5')
+    ap.add_argument('--plain', action='store_true',
+                    help='headline kernels only, a few launches each, no cache flush (for profiler runs)')
     ap.add_argument('--traffic-probe', action='store_true',
                     help='also run one elementwise kernel of known HBM traffic (256 MiB read + 256 MiB '
                          'written) so that FETCH_SIZE / WRITE_SIZE counters can be scaled')
+    ap.add_argument('--mfma-peak', action='store_true',
+                    help='only measure what the matrix pipe sustains (register-only MFMA loop, constant '
+                         'and random operands) and print that as one JSON line')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU only (attention shards by batch/head with no '
               'exchange); use --gpus 1', file=sys.stderr)
         sys.exit(2)
 
+    import numpy as np
     import torch
     from aotriton_amd import flash
+    from aotriton_amd._lib import lib
     from aotriton_amd.pyaotriton.v3.flash import attn_bwd_kernel, attn_bwd_params
 
     dev = torch.device('cuda', 0)
     torch.cuda.set_device(dev)
     props = torch.cuda.get_device_properties(0)
+    stream_ptr = flash._stream().native() or None
+    device = {'name': props.name, 'multiProcessorCount': lib.fa_get_multiprocessor_count(stream_ptr),
+              'clock_rate_khz': lib.fa_get_clock_rate_khz(stream_ptr)}
+    ok = flash.hipError_t.hipSuccess
+    tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
+    flush = torch.empty(FLUSH_BYTES, device=dev, dtype=torch.int8)
+
+    def do_bench(fn, warmup_ms=25.0, rep_ms=100.0, max_reps=400):
+        """Per-launch times of fn (ms): {'median','p20','p80','mean','reps'}."""
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            fn()
+        e1.record()
+        e1.synchronize()
+        est = max(e0.elapsed_time(e1) / 3, 1e-3)
+        for _ in range(max(1, int(warmup_ms / est))):
+            fn()
+        n = max(5, min(max_reps, int(math.ceil(rep_ms / est))))
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+        for i in range(n):
+            flush.zero_()
+            starts[i].record()
+            fn()
+            ends[i].record()
+        torch.cuda.synchronize()
+        t = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+        q = lambda p: t[min(n - 1, int(p * n))]
+        return {'median': q(0.5), 'p20': q(0.2), 'p80': q(0.8), 'mean': sum(t) / n, 'reps': n}
+
+    if args.mfma_peak:
+        grid, iters = 512, 40000
+        out = torch.empty(grid * 256, device=dev, dtype=torch.float32)
+        clk = torch.zeros(2, device=dev, dtype=torch.int64)
+        res = {}
+        for name, rnd in (('constant_operands', 0), ('random_operands', 1)):
+            run = lambda: lib.fa_probe_mfma_rate(rnd, grid, iters, out.data_ptr(), clk.data_ptr(), stream_ptr)
+            assert run() == 0
+            r = do_bench(run, warmup_ms=50.0, rep_ms=200.0, max_reps=8)
+            c = clk.cpu().tolist()
+            fl = grid * 4.0 * iters * 32 * 32768.0
+            res[name] = {'ms': r['median'], 'tflops': tf(fl, r['median']),
+                         'shader_clock_ghz': c[0] / (c[1] / 100e6) / 1e9 if c[1] else None}
+        print(json.dumps({'metric': 'sustained v_mfma_f32_32x32x16_bf16 rate, register-only loop', 'unit': 'TFLOPS',
+                          'device': device, 'peak_tflops_used': PEAK_BF16_TFLOPS, **res}))
+        return
+
     B, H, S, D = 4, 32, 4096, 128
     causal = True
     dtype = torch.bfloat16
@@ -103,7 +177,6 @@ def main():
     null = torch.empty([0], device=dev, dtype=torch.uint64)
     atomic = torch.zeros([1], device=dev, dtype=torch.int32)
     sm = 1.0 / math.sqrt(D)
-    ok = flash.hipError_t.hipSuccess
 
     def fwd():
         atomic.zero_()
@@ -120,17 +193,6 @@ def main():
 
     def bwd_slot(slot):
         assert attn_bwd_kernel(bparams, attn_bwd_params.kVersion, flash._stream(), slot) == ok
-
-    def timed(fn, n):
-        """Average duration (ms) of fn over n launches, HIP events on the launch stream."""
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(n):
-            fn()
-        e1.record()
-        e1.synchronize()
-        return e0.elapsed_time(e1) / n
 
     if args.traffic_probe:
         x = torch.zeros(64 * 1024 * 1024, device=dev, dtype=torch.float32)
@@ -152,32 +214,56 @@ def main():
         bwd(0)
     torch.cuda.synchronize()
     step_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    if args.plain:
+        for slot in (0, 1, 2, 3):
+            for _ in range(3):
+                bwd_slot(slot)
+        torch.cuda.synchronize()
+        print(json.dumps({'plain': True, 'ms_per_step': step_ms, 'steps': args.steps}))
+        return
 
-    n = max(args.steps, 5)
-    t_fwd = timed(fwd, n)
-    t_split = timed(lambda: bwd(0), n)
-    t_fused = timed(lambda: bwd(1), n)
-    t_pre = timed(lambda: bwd_slot(0), n)
-    t_dkdv = timed(lambda: bwd_slot(1), n)
-    t_dq = timed(lambda: bwd_slot(2), n)
+    r_fwd = do_bench(fwd)
+    r_split = do_bench(lambda: bwd(0))
+    r_fused = do_bench(lambda: bwd(1))
+    r_pre = do_bench(lambda: bwd_slot(0))
+    r_dkdv = do_bench(lambda: bwd_slot(1))
+    r_dq = do_bench(lambda: bwd_slot(2))
     torch.cuda.synchronize()
 
     f_fwd = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
     f_bwd = 2.5 * f_fwd
-    tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
     value = tf(f_fwd + f_bwd, step_ms)
+
+    def row(fl, r, extra=None):
+        d = {'ms': r['median'], 'ms_p20': r['p20'], 'ms_p80': r['p80'], 'reps': r['reps'],
+             'tflops': tf(fl, r['median']), 'frac_peak': tf(fl, r['median']) / PEAK_BF16_TFLOPS}
+        if extra:
+            d.update(extra)
+        return d
 
     # Dominant kernel of the step and the GEMM work it is required to do:
     # forward 2 GEMMs, dK/dV 4 GEMMs (S, dP, dV, dK), dQ 3 GEMMs (S, dP, dQ); one
     # causal GEMM = 2*B*H*S^2*D*0.5 FLOP.
     gemm = 2.0 * B * H * S * S * D * (0.5 if causal else 1.0)
-    kernels = {'fwd_kernel': (t_fwd, 2 * gemm), 'bwd_dkdv_kernel': (t_dkdv, 4 * gemm),
-               'bwd_dq_kernel': (t_dq, 3 * gemm)}
-    dom = max(kernels, key=lambda kname: kernels[kname][0])
-    dom_ms, dom_fl = kernels[dom]
+    kernels = {'fwd_kernel': (r_fwd, 2 * gemm), 'bwd_dkdv_kernel': (r_dkdv, 4 * gemm),
+               'bwd_dq_kernel': (r_dq, 3 * gemm)}
+    dom = max(kernels, key=lambda kname: kernels[kname][0]['mean'])
+    dom_r, dom_fl = kernels[dom]
+    dom_ms = dom_r['mean']
+    # the backward as a whole in the reference's convention (5 GEMMs of algorithmic work, 7 executed)
+    bwd_kernels_ms = r_pre['mean'] + r_dkdv['mean'] + r_dq['mean']
+    elem = 2 * B * H * S * D                                   # bytes of one bf16 activation tensor
+    algorithmic_bytes = {'fwd_kernel': 4 * elem + 4 * B * H * S,            # Q, K, V in, O out, LSE out
+                         'bwd_dkdv_kernel': 6 * elem + 8 * B * H * S,       # Q, K, V, dO in, dK, dV out, LSE, delta in
+                         'bwd_dq_kernel': 5 * elem + 8 * B * H * S}         # Q, K, V, dO in, dQ out, LSE, delta in
     roofline = {'bound': 'mfma', 'kernel': dom, 'achieved': tf(dom_fl, dom_ms), 'peak': PEAK_BF16_TFLOPS,
                 'unit': 'TFLOP/s', 'frac': tf(dom_fl, dom_ms) / PEAK_BF16_TFLOPS,
-                'traffic': HBM_BYTES_PER_LAUNCH.get(dom), 'avg_ms': dom_ms, 'flop_per_launch': dom_fl}
+                'traffic': hbm_bytes_from_profile(dom), 'algorithmic_bytes': algorithmic_bytes[dom],
+                'avg_ms': dom_ms, 'median_ms': dom_r['median'], 'flop_per_launch': dom_fl,
+                'frac_ref_convention': tf(f_bwd, bwd_kernels_ms) / PEAK_BF16_TFLOPS,
+                'frac_ref_convention_note': 'whole split backward: 2.5 x forward FLOP (5 GEMMs) over the summed '
+                                            'mean durations of its three kernels; frac counts the GEMMs the '
+                                            'dominant kernel executes'}
 
     out = {
         'metric': 'attn fwd/bwd TFLOPS and % bf16 MFMA peak, B4 H32 S4096 D128 causal, 1 GPU',
@@ -187,14 +273,84 @@ def main():
         'config': {'workload': 'attention fwd + bwd(split), B=4 Hq=Hkv=32 Sq=Sk=4096 D=128 bf16 causal, '
                                'q,k,v,dO~N(0,1) seed 1234, sm_scale=1/sqrt(128)'},
         'peak_tflops_used': PEAK_BF16_TFLOPS,
-        'device': {'name': props.name, 'multiProcessorCount': props.multi_processor_count,
-                   'clock_rate_khz': getattr(props, 'clock_rate', None)},
-        'fwd': {'ms': t_fwd, 'tflops': tf(f_fwd, t_fwd), 'frac_peak': tf(f_fwd, t_fwd) / PEAK_BF16_TFLOPS},
-        'bwd_split': {'ms': t_split, 'tflops': tf(f_bwd, t_split), 'frac_peak': tf(f_bwd, t_split) / PEAK_BF16_TFLOPS,
-                      'kernels_ms': {'bwd_preprocess': t_pre, 'bwd_dkdv': t_dkdv, 'bwd_dq': t_dq}},
-        'bwd_fused': {'ms': t_fused, 'tflops': tf(f_bwd, t_fused), 'frac_peak': tf(f_bwd, t_fused) / PEAK_BF16_TFLOPS},
+        'device': device,
+        'timing': 'per launch: 512 MiB zeroed before it, warm-up >= 25 ms, >= 100 ms of launches, HIP events, '
+                  'median (p20, p80); value/ms_per_step: K back-to-back steps between synchronisations',
+        'fwd': row(f_fwd, r_fwd),
+        'bwd_split': row(f_bwd, r_split, {'kernels_ms': {'bwd_preprocess': r_pre['median'], 'bwd_dkdv': r_dkdv['median'],
+                                                         'bwd_dq': r_dq['median']}}),
+        'bwd_fused': row(f_bwd, r_fused),
         'roofline': roofline,
     }
+
+    if not args.no_extra:
+        del q, k, v, do, o, dq, dk, dv
+        torch.cuda.empty_cache()
+        # --- configuration 4: GQA, 16 packed sequences U[256, 8192], causal, bf16, D=128 -------------
+        rng = np.random.default_rng(seed)
+        lens = rng.integers(256, 8193, size=16)
+        cu = np.zeros(17, dtype=np.int32)
+        cu[1:] = np.cumsum(lens)
+        T, Hq, Hk = int(cu[-1]), 32, 8
+        gg = torch.Generator(device=dev).manual_seed(seed)
+        mk = lambda h: torch.randn(1, T, h, 128, device=dev, dtype=torch.float32, generator=gg).to(torch.bfloat16).transpose(1, 2)
+        q4, k4, v4, do4 = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+        o4, dq4, dk4, dv4 = torch.empty_like(q4), torch.empty_like(q4), torch.empty_like(k4), torch.empty_like(v4)
+        L4 = torch.empty(Hq, T, device=dev, dtype=torch.float32)
+        d4 = torch.empty_like(L4)
+        cuq = torch.from_numpy(cu).to(dev)
+        mx = int(lens.max())
+        sm4 = 1.0 / math.sqrt(128)
+
+        def fwd4():
+            atomic.zero_()
+            assert flash.attn_fwd_compact_varlen(q4, k4, v4, None, cuq, cuq, mx, mx, sm4, L4, o4, 0.0, null, null, 0,
+                                                 null, null, None, True, atomic) == ok
+
+        def bwd4():
+            assert flash.attn_bwd_compact_varlen(q4, k4, v4, cuq, cuq, mx, mx, None, sm4, o4, do4, dq4, dk4, dv4, None,
+                                                 L4, d4, 0.0, null, null, 0, True) == ok
+
+        fl4 = sum(4.0 * Hq * float(s) ** 2 * 128 * 0.5 for s in lens)
+        out['c4'] = {'workload': f'GQA Hq=32 Hkv=8 D=128 bf16 causal, 16 packed sequences U[256,8192] (seed {seed}), '
+                                 f'{T} tokens, THD storage',
+                     'fwd': row(fl4, do_bench(fwd4)), 'bwd_split': row(2.5 * fl4, do_bench(bwd4))}
+        del q4, k4, v4, do4, o4, dq4, dk4, dv4
+        torch.cuda.empty_cache()
+        # --- configuration 5: B2 H16 S8192 D256 fp16, window (1024, 0) + bias + dropout 0.1 ----------
+        B5, H5, S5, D5 = 2, 16, 8192, 256
+        rn5 = lambda *s, sc=1.0: (torch.randn(*s, device=dev, dtype=torch.float32, generator=gg) * sc).to(torch.float16)
+        q5, k5, v5, do5 = (rn5(B5, H5, S5, D5) for _ in range(4))
+        b5 = torch.empty(B5, H5, S5, S5, device=dev, dtype=torch.float16)
+        for i in range(B5):
+            for h in range(H5):
+                b5[i, h] = rn5(S5, S5, sc=0.5)
+        o5, dq5, dk5, dv5 = torch.empty_like(q5), torch.empty_like(q5), torch.empty_like(k5), torch.empty_like(v5)
+        db5 = torch.empty_like(b5)
+        L5 = torch.empty(B5 * H5, S5, device=dev, dtype=torch.float32)
+        d5 = torch.empty_like(L5)
+        u64 = lambda x: torch.tensor([x], device=dev, dtype=torch.uint64)
+        seed5, off5, so5, oo5 = u64(0x1234), u64(0), u64(0), u64(0)
+        sm5 = 1.0 / math.sqrt(D5)
+
+        def fwd5():
+            atomic.zero_()
+            assert flash.attn_fwd(q5, k5, v5, b5, sm5, L5, o5, 0.1, seed5, off5, 0, so5, oo5, None, (1024, 0), atomic) == ok
+
+        def bwd5(with_db):
+            assert flash.attn_bwd(q5, k5, v5, b5, sm5, o5, do5, dq5, dk5, dv5, db5 if with_db else None, None, L5, d5,
+                                  0.1, so5, oo5, 0, (1024, 0)) == ok
+
+        fl5 = 4.0 * B5 * H5 * D5 * 7872000.0          # visible (query, key) pairs per head: sum_i (min(i, 1024) + 1)
+        out['c5'] = {'workload': 'B=2 H=16 S=8192 D=256 fp16, window (1024, 0), bias (B,H,S,S) ~ N(0,0.5), dropout 0.1 '
+                                 'seed 0x1234 offset 0',
+                     'fwd': row(fl5, do_bench(fwd5, max_reps=100)),
+                     'bwd_split_no_db': row(2.5 * fl5, do_bench(lambda: bwd5(False), max_reps=60)),
+                     'bwd_split_with_db': row(2.5 * fl5, do_bench(lambda: bwd5(True), max_reps=60),
+                                              {'note': 'dB is a dense (B,H,S,S) tensor: 4 GiB written, zeros outside the band'})}
+        del q5, k5, v5, do5, b5, db5
+        torch.cuda.empty_cache()
+
     if not args.no_cpu:
         out['cpu_baseline'] = cpu_baseline(B, H, S, D, causal, seed)
     print(json.dumps(out))
