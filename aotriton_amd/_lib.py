@@ -98,6 +98,25 @@ SYMBOLS = {
     'fa_check_gpu': (ctypes.c_int, [ctypes.c_void_p]),
     'fa_attn_fwd': (ctypes.c_int, [P(fa_fwd_params), ctypes.c_int32, ctypes.c_void_p, P(fa_options)]),
     'fa_attn_bwd': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p, P(fa_options)]),
+    'fa_v2_attn_fwd': (ctypes.c_int, [P(fa_tensor4)] * 4 + [ctypes.c_float, P(fa_tensor2), P(fa_tensor4), ctypes.c_float,
+                                      P(fa_tensor0), P(fa_tensor0), ctypes.c_int64, P(fa_tensor0), P(fa_tensor0),
+                                      P(fa_tensor4), ctypes.c_int32, P(fa_tensor0), ctypes.c_void_p]),
+    'fa_v2_attn_fwd_compact_varlen': (ctypes.c_int, [P(fa_tensor4)] * 4 + [P(fa_tensor1), P(fa_tensor1), ctypes.c_int32,
+                                                     ctypes.c_int32, ctypes.c_float, P(fa_tensor2), P(fa_tensor4),
+                                                     ctypes.c_float, P(fa_tensor0), P(fa_tensor0), ctypes.c_int64,
+                                                     P(fa_tensor0), P(fa_tensor0), P(fa_tensor4), ctypes.c_int32,
+                                                     P(fa_tensor0), ctypes.c_void_p]),
+    'fa_v2_attn_bwd': (ctypes.c_int, [P(fa_tensor4)] * 4 + [ctypes.c_float] + [P(fa_tensor4)] * 6 +
+                       [P(fa_tensor2), P(fa_tensor2), ctypes.c_float, P(fa_tensor0), P(fa_tensor0), ctypes.c_int64,
+                        ctypes.c_int32, ctypes.c_void_p]),
+    'fa_v2_attn_bwd_fused': (ctypes.c_int, [P(fa_tensor4)] * 4 + [ctypes.c_float] + [P(fa_tensor4)] * 6 +
+                             [P(fa_tensor2), ctypes.c_float, P(fa_tensor0), P(fa_tensor0), ctypes.c_int64,
+                              ctypes.c_int32, ctypes.c_void_p]),
+    'fa_v2_attn_bwd_compact_varlen': (ctypes.c_int, [P(fa_tensor4)] * 3 + [P(fa_tensor1), P(fa_tensor1), ctypes.c_int32,
+                                                     ctypes.c_int32, P(fa_tensor4), ctypes.c_float] +
+                                      [P(fa_tensor4)] * 6 + [P(fa_tensor2), P(fa_tensor2), ctypes.c_float,
+                                                             P(fa_tensor0), P(fa_tensor0), ctypes.c_int64,
+                                                             ctypes.c_int32, ctypes.c_void_p]),
     'fa_attn_bwd_noalloc': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p]),
     'fa_attn_bwd_kernel': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32]),
     'fa_debug_simulate_encoded_softmax': (ctypes.c_int, [P(fa_tensor4), ctypes.c_float, P(fa_tensor0),

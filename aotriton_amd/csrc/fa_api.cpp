@@ -657,6 +657,133 @@ int fa_attn_bwd(const fa_bwd_params* p, int32_t params_version, void* hip_stream
   return attn_bwd_impl(p, params_version, hip_stream, options, -1);
 }
 
+// ---- v2 positional entry points ------------------------------------------------------------
+// Thin fills of the v3 params: is_causal -> windowed with the top-left sentinels, compact
+// packed sequences -> varlen_type 1 (the reference's Python layer does the same,
+// modules/flash/tests/aotriton_flash.py:141-196,277-335).
+
+extern "C++" {
+namespace {
+template <typename V> V view_or_null(const V* t) { return t ? *t : V{}; }
+
+void set_causal(bool is_causal, int8_t* type, int32_t* left, int32_t* right) {
+  *type = is_causal ? FA_CAUSAL_WINDOWED : FA_CAUSAL_NONE;
+  *left = *right = is_causal ? FA_WINDOW_TOP_LEFT : 0;
+}
+
+int v2_fwd(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor4* b,
+           const fa_tensor1* cu_q, const fa_tensor1* cu_k, int32_t max_sq, int32_t max_sk, float sm_scale,
+           const fa_tensor2* lse, const fa_tensor4* out, float dropout_p, const fa_tensor0* seed,
+           const fa_tensor0* off1, int64_t off2, const fa_tensor0* seed_out, const fa_tensor0* off_out,
+           const fa_tensor4* encoded_softmax, int32_t is_causal, const fa_tensor0* atomic, void* stream) {
+  if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERROR_INVALID_VALUE;
+  fa_fwd_params p{};
+  p.Q = *q; p.K = *k; p.V = *v; p.B = view_or_null(b);
+  p.Sm_scale = sm_scale;
+  p.L = view_or_null(lse);
+  p.Out = *out;
+  p.cu_seqlens_q = view_or_null(cu_q); p.cu_seqlens_k = view_or_null(cu_k);
+  p.Max_seqlen_q = max_sq; p.Max_seqlen_k = max_sk;
+  p.varlen_type = cu_q != nullptr ? FA_VARLEN_COMPACT : FA_VARLEN_NONE;
+  p.dropout_p = dropout_p;
+  p.philox_seed_ptr = view_or_null(seed); p.philox_offset1 = view_or_null(off1);
+  p.philox_offset2 = (uint64_t)off2;
+  p.philox_seed_output = view_or_null(seed_out); p.philox_offset_output = view_or_null(off_out);
+  p.encoded_softmax = view_or_null(encoded_softmax);
+  p.persistent_atomic_counter = view_or_null(atomic);
+  set_causal(is_causal != 0, &p.causal_type, &p.window_left, &p.window_right);
+  return fa_attn_fwd(&p, FA_FWD_PARAMS_VERSION, stream, nullptr);
+}
+
+int v2_bwd(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor4* b,
+           const fa_tensor1* cu_q, const fa_tensor1* cu_k, int32_t max_sq, int32_t max_sk, float sm_scale,
+           const fa_tensor4* out, const fa_tensor4* dout, const fa_tensor4* dq, const fa_tensor4* dk,
+           const fa_tensor4* dv, const fa_tensor4* db, const fa_tensor2* lse, const fa_tensor2* delta,
+           float dropout_p, const fa_tensor0* seed, const fa_tensor0* off1, int64_t off2, int32_t is_causal,
+           int backend, void* stream) {
+  if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || dout == nullptr || dq == nullptr ||
+      dk == nullptr || dv == nullptr || lse == nullptr)
+    return FA_ERROR_INVALID_VALUE;
+  fa_bwd_params p{};
+  p.Q = *q; p.K = *k; p.V = *v; p.B = view_or_null(b);
+  p.Sm_scale = sm_scale;
+  p.Out = *out; p.DO = *dout; p.DQ = *dq; p.DK = *dk; p.DV = *dv; p.DB = view_or_null(db);
+  p.L = *lse;
+  p.D.eager = view_or_null(delta);
+  p.cu_seqlens_q = view_or_null(cu_q); p.cu_seqlens_k = view_or_null(cu_k);
+  p.Max_seqlen_q = max_sq; p.Max_seqlen_k = max_sk;
+  p.varlen_type = cu_q != nullptr ? FA_VARLEN_COMPACT : FA_VARLEN_NONE;
+  p.dropout_p = dropout_p;
+  p.philox_seed_ptr = view_or_null(seed); p.philox_offset1 = view_or_null(off1);
+  p.philox_offset2 = (uint64_t)off2;
+  set_causal(is_causal != 0, &p.causal_type, &p.window_left, &p.window_right);
+  fa_options opt{backend, 0};
+  return fa_attn_bwd(&p, FA_BWD_PARAMS_VERSION, stream, &opt);
+}
+}  // namespace
+}  // extern "C++"
+
+int fa_v2_attn_fwd(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor4* b,
+                   float sm_scale, const fa_tensor2* softmax_lse, const fa_tensor4* out, float dropout_p,
+                   const fa_tensor0* philox_seed, const fa_tensor0* philox_offset1, int64_t philox_offset2,
+                   const fa_tensor0* philox_seed_output, const fa_tensor0* philox_offset_output,
+                   const fa_tensor4* encoded_softmax, int32_t is_causal, const fa_tensor0* atomic_for_causal,
+                   void* hip_stream) {
+  return v2_fwd(q, k, v, b, nullptr, nullptr, 0, 0, sm_scale, softmax_lse, out, dropout_p, philox_seed,
+                philox_offset1, philox_offset2, philox_seed_output, philox_offset_output, encoded_softmax,
+                is_causal, atomic_for_causal, hip_stream);
+}
+
+int fa_v2_attn_fwd_compact_varlen(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v,
+                                  const fa_tensor4* b, const fa_tensor1* cu_seqlens_q,
+                                  const fa_tensor1* cu_seqlens_k, int32_t max_seqlen_q, int32_t max_seqlen_k,
+                                  float sm_scale, const fa_tensor2* softmax_lse, const fa_tensor4* out,
+                                  float dropout_p, const fa_tensor0* philox_seed,
+                                  const fa_tensor0* philox_offset1, int64_t philox_offset2,
+                                  const fa_tensor0* philox_seed_output, const fa_tensor0* philox_offset_output,
+                                  const fa_tensor4* encoded_softmax, int32_t is_causal,
+                                  const fa_tensor0* atomic_for_causal, void* hip_stream) {
+  if (cu_seqlens_q == nullptr || cu_seqlens_k == nullptr) return FA_ERROR_INVALID_VALUE;
+  return v2_fwd(q, k, v, b, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale, softmax_lse, out,
+                dropout_p, philox_seed, philox_offset1, philox_offset2, philox_seed_output, philox_offset_output,
+                encoded_softmax, is_causal, atomic_for_causal, hip_stream);
+}
+
+int fa_v2_attn_bwd(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor4* b,
+                   float sm_scale, const fa_tensor4* out, const fa_tensor4* dout, const fa_tensor4* dq,
+                   const fa_tensor4* dk, const fa_tensor4* dv, const fa_tensor4* db,
+                   const fa_tensor2* softmax_lse, const fa_tensor2* delta, float dropout_p,
+                   const fa_tensor0* philox_seed, const fa_tensor0* philox_offset1, int64_t philox_offset2,
+                   int32_t is_causal, void* hip_stream) {
+  if (delta == nullptr) return FA_ERROR_INVALID_VALUE;
+  return v2_bwd(q, k, v, b, nullptr, nullptr, 0, 0, sm_scale, out, dout, dq, dk, dv, db, softmax_lse, delta,
+                dropout_p, philox_seed, philox_offset1, philox_offset2, is_causal, 0, hip_stream);
+}
+
+int fa_v2_attn_bwd_fused(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor4* b,
+                         float sm_scale, const fa_tensor4* out, const fa_tensor4* dout, const fa_tensor4* dq,
+                         const fa_tensor4* dk, const fa_tensor4* dv, const fa_tensor4* db,
+                         const fa_tensor2* softmax_lse, float dropout_p, const fa_tensor0* philox_seed,
+                         const fa_tensor0* philox_offset1, int64_t philox_offset2, int32_t is_causal,
+                         void* hip_stream) {
+  return v2_bwd(q, k, v, b, nullptr, nullptr, 0, 0, sm_scale, out, dout, dq, dk, dv, db, softmax_lse, nullptr,
+                dropout_p, philox_seed, philox_offset1, philox_offset2, is_causal, 1, hip_stream);
+}
+
+int fa_v2_attn_bwd_compact_varlen(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v,
+                                  const fa_tensor1* cu_seqlens_q, const fa_tensor1* cu_seqlens_k,
+                                  int32_t max_seqlen_q, int32_t max_seqlen_k, const fa_tensor4* b, float sm_scale,
+                                  const fa_tensor4* out, const fa_tensor4* dout, const fa_tensor4* dq,
+                                  const fa_tensor4* dk, const fa_tensor4* dv, const fa_tensor4* db,
+                                  const fa_tensor2* softmax_lse, const fa_tensor2* delta, float dropout_p,
+                                  const fa_tensor0* philox_seed, const fa_tensor0* philox_offset1,
+                                  int64_t philox_offset2, int32_t is_causal, void* hip_stream) {
+  if (cu_seqlens_q == nullptr || cu_seqlens_k == nullptr || delta == nullptr) return FA_ERROR_INVALID_VALUE;
+  return v2_bwd(q, k, v, b, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale, out, dout, dq, dk,
+                dv, db, softmax_lse, delta, dropout_p, philox_seed, philox_offset1, philox_offset2, is_causal, 0,
+                hip_stream);
+}
+
 int fa_attn_bwd_noalloc(const fa_bwd_params* p, int32_t params_version, void* hip_stream) {
   return attn_bwd_impl(p, params_version, hip_stream, nullptr, -1, true);
 }

@@ -158,3 +158,64 @@ def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.
     o, _ = torch.ops.aotriton_amd.flash_attention_forward(q, k, v, bias, float(dropout_p), ct, wl, wr, sm_scale,
                                                           seed, offset)
     return o
+
+
+# ---- routing torch.nn.functional.scaled_dot_product_attention itself --------------------------
+# The consumer the reference names is PyTorch's SDPA on ROCm (README.md:71-75 of the reference):
+# callers write F.scaled_dot_product_attention and the dispatcher picks the flash backend.  The
+# two hooks below give the same effect without touching callers: `sdpa_router()` is a
+# TorchFunctionMode (scoped, composes with torch.compile's tracing of the custom ops), `install()`
+# replaces the attribute on torch.nn.functional for code that cannot be wrapped in a `with`.
+def _routable(query, key, value, attn_mask, dropout_p):
+    ts = (query, key, value)
+    if not all(isinstance(t, Tensor) and t.is_cuda and t.dim() == 4 for t in ts):
+        return False
+    if query.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        return False
+    if not (key.dtype == query.dtype and value.dtype == query.dtype):
+        return False
+    dqk, dv = query.shape[-1], value.shape[-1]
+    if dqk % 8 or dv % 8 or dqk > 512 or dv > 512 or key.shape[-1] != dqk:
+        return False
+    if query.shape[1] % max(key.shape[1], 1) or key.shape[1] != value.shape[1]:
+        return False
+    if attn_mask is not None and not isinstance(attn_mask, Tensor):
+        return False
+    if getattr(query, 'is_nested', False) or getattr(key, 'is_nested', False):
+        return False
+    return True
+
+
+_torch_sdpa = torch.nn.functional.scaled_dot_product_attention
+
+
+def _dispatch(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, enable_gqa=False):
+    if _routable(query, key, value, attn_mask, dropout_p):
+        gqa = enable_gqa or query.shape[1] != key.shape[1]
+        return scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal, scale, gqa)
+    return _torch_sdpa(query, key, value, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal,
+                       scale=scale, enable_gqa=enable_gqa)
+
+
+class sdpa_router(torch.overrides.TorchFunctionMode):
+    """`with sdpa_router(): ...` sends every F.scaled_dot_product_attention call on 4-D CUDA
+    fp16/bf16/fp32 tensors (head dims multiples of 8 up to 512) to this library's operators;
+    anything else falls through to PyTorch's own implementation."""
+
+    def __torch_function__(self, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        if func is _torch_sdpa:
+            with torch._C.DisableTorchFunction():
+                return _dispatch(*args, **kwargs)
+        return func(*args, **kwargs)
+
+
+def install():
+    """Make torch.nn.functional.scaled_dot_product_attention route here process-wide
+    (undo with uninstall()).  Modules that bound the function at import time keep the original;
+    for those use the sdpa_router() mode."""
+    torch.nn.functional.scaled_dot_product_attention = _dispatch
+
+
+def uninstall():
+    torch.nn.functional.scaled_dot_product_attention = _torch_sdpa

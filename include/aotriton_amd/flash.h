@@ -217,6 +217,51 @@ FA_API int fa_attn_fwd(const fa_fwd_params* params, int32_t params_version,
 FA_API int fa_attn_bwd(const fa_bwd_params* params, int32_t params_version,
                        void* hip_stream, const fa_options* options);
 
+/* The positional v2 API: v2::flash::attn_fwd, attn_fwd_compact_varlen, attn_bwd, attn_bwd_fused,
+ * attn_bwd_compact_varlen.  These are not in the reference tree (0.14 keeps only the v3 params
+ * entry points); their signatures are those of AOTriton 0.11's include/aotriton/v2/flash.h:31-141
+ * as shipped inside PyTorch, with views passed by pointer (null = the reference's empty view),
+ * bool as int32 and the extra-arguments pointer dropped.  Each fills the v3 params: is_causal
+ * becomes causal_type 3 with the top-left sentinels, cu_seqlens make varlen_type 1.  attn_bwd runs
+ * the split backend, attn_bwd_fused the single-launch backend. */
+FA_API int fa_v2_attn_fwd(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v,
+                          const fa_tensor4* b, float sm_scale, const fa_tensor2* softmax_lse,
+                          const fa_tensor4* out, float dropout_p, const fa_tensor0* philox_seed,
+                          const fa_tensor0* philox_offset1, int64_t philox_offset2,
+                          const fa_tensor0* philox_seed_output,
+                          const fa_tensor0* philox_offset_output,
+                          const fa_tensor4* encoded_softmax, int32_t is_causal,
+                          const fa_tensor0* atomic_for_causal, void* hip_stream);
+FA_API int fa_v2_attn_fwd_compact_varlen(
+    const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor4* b,
+    const fa_tensor1* cu_seqlens_q, const fa_tensor1* cu_seqlens_k, int32_t max_seqlen_q,
+    int32_t max_seqlen_k, float sm_scale, const fa_tensor2* softmax_lse, const fa_tensor4* out,
+    float dropout_p, const fa_tensor0* philox_seed, const fa_tensor0* philox_offset1,
+    int64_t philox_offset2, const fa_tensor0* philox_seed_output,
+    const fa_tensor0* philox_offset_output, const fa_tensor4* encoded_softmax, int32_t is_causal,
+    const fa_tensor0* atomic_for_causal, void* hip_stream);
+FA_API int fa_v2_attn_bwd(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v,
+                          const fa_tensor4* b, float sm_scale, const fa_tensor4* out,
+                          const fa_tensor4* dout, const fa_tensor4* dq, const fa_tensor4* dk,
+                          const fa_tensor4* dv, const fa_tensor4* db, const fa_tensor2* softmax_lse,
+                          const fa_tensor2* delta, float dropout_p, const fa_tensor0* philox_seed,
+                          const fa_tensor0* philox_offset1, int64_t philox_offset2,
+                          int32_t is_causal, void* hip_stream);
+FA_API int fa_v2_attn_bwd_fused(const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v,
+                                const fa_tensor4* b, float sm_scale, const fa_tensor4* out,
+                                const fa_tensor4* dout, const fa_tensor4* dq, const fa_tensor4* dk,
+                                const fa_tensor4* dv, const fa_tensor4* db,
+                                const fa_tensor2* softmax_lse, float dropout_p,
+                                const fa_tensor0* philox_seed, const fa_tensor0* philox_offset1,
+                                int64_t philox_offset2, int32_t is_causal, void* hip_stream);
+FA_API int fa_v2_attn_bwd_compact_varlen(
+    const fa_tensor4* q, const fa_tensor4* k, const fa_tensor4* v, const fa_tensor1* cu_seqlens_q,
+    const fa_tensor1* cu_seqlens_k, int32_t max_seqlen_q, int32_t max_seqlen_k, const fa_tensor4* b,
+    float sm_scale, const fa_tensor4* out, const fa_tensor4* dout, const fa_tensor4* dq,
+    const fa_tensor4* dk, const fa_tensor4* dv, const fa_tensor4* db, const fa_tensor2* softmax_lse,
+    const fa_tensor2* delta, float dropout_p, const fa_tensor0* philox_seed,
+    const fa_tensor0* philox_offset1, int64_t philox_offset2, int32_t is_causal, void* hip_stream);
+
 /* The split backward for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): same inputs, outputs and
  * results as fa_attn_bwd with backend 0, but delta lives in a device array that belongs to

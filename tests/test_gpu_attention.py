@@ -5,6 +5,8 @@ oracle run in fp32 on the same seeded inputs.  Tolerances are the reference's
 GQA, BSHD strides, causal on/off, dropout on/off, fp16/bf16."""
 import math
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -470,3 +472,68 @@ def test_sdpa_entry_point_matches_torch_math(mode):
     check('out', outs[0], outs[1], outs[2], FUDGE['out'])
     for name, i in (('dq', 0), ('dk', 1), ('dv', 2)):
         check(name, grads[0][i], grads[1][i], grads[2][i], FUDGE[name])
+
+
+@pytest.mark.gpu
+def test_v2_positional_c_abi_matches_the_params_entry_points():
+    """fa_v2_attn_fwd / attn_bwd / attn_bwd_fused / *_compact_varlen against fa_attn_fwd / fa_attn_bwd
+    on the same inputs: bit-identical O, LSE, dQ, dK, dV."""
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton.v2 import flash as v2
+    mk = flash.mk_aotensor
+    ok = flash.hipError_t.hipSuccess
+    s = flash._stream()
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    B, Hq, Hk, Sq, Sk, D = 2, 4, 2, 300, 421, 128
+    q, k, v, _, do = make_inputs(B, Hq, Hk, Sq, Sk, D, torch.bfloat16, DEV, seed=5)
+    sm = 1.0 / math.sqrt(D)
+    for causal in (False, True):
+        o1, o2 = torch.empty_like(q), torch.empty_like(q)
+        L1 = torch.empty(B * Hq, Sq, device=DEV, dtype=torch.float32)
+        L2 = torch.empty_like(L1)
+        atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+        assert flash.attn_fwd(q, k, v, None, sm, L1, o1, 0.0, null, null, 0, null, null, None, causal, atomic) == ok
+        assert v2.attn_fwd(mk(q), mk(k), mk(v), None, sm, mk(L2), mk(o2), 0.0, None, None, 0, None, None, None, causal,
+                           mk(atomic), s) == ok
+        assert torch.equal(o1, o2) and torch.equal(L1, L2)
+        for fused in (False, True):
+            g1 = [torch.empty_like(t) for t in (q, k, v)]
+            g2 = [torch.empty_like(t) for t in (q, k, v)]
+            delta = torch.empty_like(L1)
+            ext = flash.attn_options()
+            ext.force_backend_index = 1 if fused else 0
+            assert flash.attn_bwd(q, k, v, None, sm, o1, do, g1[0], g1[1], g1[2], None, None, L1, delta, 0.0, null, null,
+                                  0, causal, extargs=ext) == ok
+            if fused:
+                assert v2.attn_bwd_fused(mk(q), mk(k), mk(v), None, sm, mk(o1), mk(do), mk(g2[0]), mk(g2[1]), mk(g2[2]),
+                                         None, mk(L1), 0.0, None, None, 0, causal, s) == ok
+            else:
+                assert v2.attn_bwd(mk(q), mk(k), mk(v), None, sm, mk(o1), mk(do), mk(g2[0]), mk(g2[1]), mk(g2[2]), None,
+                                   mk(L1), mk(delta), 0.0, None, None, 0, causal, s) == ok
+            for a, b in zip(g1, g2):
+                assert torch.equal(a, b)
+    # packed sequences
+    lens = [100, 37, 256]
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=DEV)
+    T = sum(lens)
+    qv, kv, vv, _, dov = make_inputs(1, Hq, Hk, T, T, D, torch.bfloat16, DEV, seed=6, bshd=True)
+    o1, o2 = torch.empty_like(qv), torch.empty_like(qv)
+    L1 = torch.empty(Hq, T, device=DEV, dtype=torch.float32)
+    L2 = torch.empty_like(L1)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+    mx = max(lens)
+    assert flash.attn_fwd_compact_varlen(qv, kv, vv, None, cu, cu, mx, mx, sm, L1, o1, 0.0, null, null, 0, null, null,
+                                         None, True, atomic) == ok
+    assert v2.attn_fwd_compact_varlen(mk(qv), mk(kv), mk(vv), None, mk(cu), mk(cu), mx, mx, sm, mk(L2), mk(o2), 0.0,
+                                      None, None, 0, None, None, None, True, mk(atomic), s) == ok
+    assert torch.equal(o1, o2) and torch.equal(L1, L2)
+    g1 = [torch.empty_like(t) for t in (qv, kv, vv)]
+    g2 = [torch.empty_like(t) for t in (qv, kv, vv)]
+    delta = torch.empty_like(L1)
+    assert flash.attn_bwd_compact_varlen(qv, kv, vv, cu, cu, mx, mx, None, sm, o1, dov, g1[0], g1[1], g1[2], None, L1,
+                                         delta, 0.0, null, null, 0, True) == ok
+    assert v2.attn_bwd_compact_varlen(mk(qv), mk(kv), mk(vv), mk(cu), mk(cu), mx, mx, None, sm, mk(o1), mk(dov),
+                                      mk(g2[0]), mk(g2[1]), mk(g2[2]), None, mk(L1), mk(delta), 0.0, None, None, 0,
+                                      True, s) == ok
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)

@@ -219,3 +219,40 @@ def test_tile_intervals_against_brute_force_and_reference_algebra():
             | (set(range(r[4], r[5] + 1)) if r[4] <= r[5] else set())
         assert ref_full <= fb
         assert {b for b in (lb | fb | rb)} <= {b for b in ref_all} | fb
+
+
+def test_v2_positional_entry_points_validate_before_any_launch():
+    """fa_v2_* fill the v3 params and go through the same host checks (views over CPU tensors,
+    every call ends in an argument error before a device is needed)."""
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton import hipError_t as E, Stream
+    from aotriton_amd.pyaotriton.v2 import flash as v2
+    mk = flash.mk_aotensor
+    B, Hq, Hk, Sq, Sk, D = 2, 4, 2, 64, 80, 128
+    dt = torch.float16
+    q = torch.zeros(B, Hq, Sq, D, dtype=dt); k = torch.zeros(B, Hk, Sk, D, dtype=dt); v = torch.zeros_like(k)
+    o = torch.zeros_like(q); L = torch.zeros(B * Hq, Sq); delta = torch.zeros_like(L)
+    s = Stream()
+    # missing tensors
+    assert v2.attn_fwd(None, mk(k), mk(v), None, 0.1, mk(L), mk(o), 0.0, None, None, 0, None, None, None, True,
+                       None, s) == E.hipErrorInvalidValue
+    assert v2.attn_bwd(mk(q), mk(k), mk(v), None, 0.1, mk(o), mk(o), mk(q), mk(k), mk(v), None, mk(L), None, 0.0,
+                       None, None, 0, False, s) == E.hipErrorInvalidValue            # split backend without delta
+    # heads of K do not divide those of Q
+    k3 = torch.zeros(B, 3, Sk, D, dtype=dt)
+    assert v2.attn_fwd(mk(q), mk(k3), mk(k3), None, 0.1, mk(L), mk(o), 0.0, None, None, 0, None, None, None, True,
+                       None, s) == E.hipErrorInvalidValue
+    # dropout without a seed, and a head dim that is not built
+    assert v2.attn_fwd(mk(q), mk(k), mk(v), None, 0.1, mk(L), mk(o), 0.5, None, None, 0, None, None, None, False,
+                       None, s) == E.hipErrorInvalidValue
+    qb = torch.zeros(B, Hq, Sq, 520, dtype=dt); kb = torch.zeros(B, Hk, Sk, 520, dtype=dt)
+    assert v2.attn_bwd_fused(mk(qb), mk(kb), mk(kb), None, 0.1, mk(qb), mk(qb), mk(qb), mk(kb), mk(kb), None, mk(L),
+                             0.0, None, None, 0, True, s) == E.hipErrorNotSupported
+    # packed sequences need both offset arrays and a batch of one
+    cu = torch.tensor([0, 30, 64], dtype=torch.int32)
+    assert v2.attn_fwd_compact_varlen(mk(q), mk(k), mk(v), None, mk(cu), None, 40, 40, 0.1, mk(L), mk(o), 0.0, None,
+                                      None, 0, None, None, None, True, None, s) == E.hipErrorInvalidValue
+    assert v2.attn_fwd_compact_varlen(mk(q), mk(k), mk(v), None, mk(cu), mk(cu), 40, 40, 0.1, mk(L), mk(o), 0.0, None,
+                                      None, 0, None, None, None, True, None, s) == E.hipErrorInvalidValue
+    assert v2.attn_bwd_compact_varlen(mk(q), mk(k), mk(v), mk(cu), mk(cu), 40, 40, None, 0.1, mk(o), mk(o), mk(q),
+                                      mk(k), mk(v), None, mk(L), None, 0.0, None, None, 0, True, s) == E.hipErrorInvalidValue

@@ -168,3 +168,55 @@ def test_forward_and_backward_replay_from_a_hip_graph(dropout_p):
         again = run()                           # eager work between replays
         torch.cuda.synchronize()
         assert torch.equal(again[0], eager[0])
+
+
+def test_router_leaves_cpu_calls_to_torch():
+    """The hooks only take CUDA tensors: on the CPU F.scaled_dot_product_attention stays torch's own."""
+    import torch.nn.functional as F
+    from aotriton_amd import torch_ops
+    q = torch.randn(1, 2, 8, 16)
+    ref = F.scaled_dot_product_attention(q, q, q, is_causal=True)
+    with torch_ops.sdpa_router():
+        assert torch.equal(F.scaled_dot_product_attention(q, q, q, is_causal=True), ref)
+    torch_ops.install()
+    try:
+        assert F.scaled_dot_product_attention is not torch_ops._torch_sdpa
+        assert torch.equal(F.scaled_dot_product_attention(q, q, q, is_causal=True), ref)
+    finally:
+        torch_ops.uninstall()
+    assert F.scaled_dot_product_attention is torch_ops._torch_sdpa
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('hook', ['mode', 'install'])
+def test_f_sdpa_routes_to_the_library(hook):
+    """F.scaled_dot_product_attention itself, unchanged call sites: under the router the library's
+    kernels run (LSE-free check: the result equals the library's own entry point bit for bit and
+    torch's math backend within tolerance), gradients included."""
+    import torch.nn.functional as F
+    from aotriton_amd import torch_ops
+    q, k, v, _, do = _inputs(B=2, Hq=4, Hk=2, Sq=200, Sk=200, D=64)
+    req = lambda t: t.detach().clone().requires_grad_()
+
+    def run(fn):
+        a, b, c = req(q), req(k), req(v)
+        o = fn(a, b, c, is_causal=True, enable_gqa=True)
+        o.backward(do)
+        return o, a.grad, b.grad, c.grad
+
+    own = run(torch_ops.scaled_dot_product_attention)
+    if hook == 'mode':
+        with torch_ops.sdpa_router():
+            routed = run(F.scaled_dot_product_attention)
+    else:
+        torch_ops.install()
+        try:
+            routed = run(F.scaled_dot_product_attention)
+        finally:
+            torch_ops.uninstall()
+    for a, b in zip(own, routed):
+        assert torch.equal(a, b)
+    with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+        ref = run(lambda a, b, c, **kw: F.scaled_dot_product_attention(a.float(), b.float(), c.float(), **kw))
+    for a, b in zip(routed, ref):
+        assert (a.float() - b).abs().max().item() < 6e-2
