@@ -472,7 +472,7 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
     case 0: out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz; break;
     case 1: out->grid[0] = persistent(grid1d(s.hk, 2, nt)); break;
     case 2: out->grid[0] = persistent(grid1d(s.hq, ratio > 2 ? (ratio > 8 ? 8 : ratio) : 2, mt)); break;
-    default: out->grid[0] = grid1d(s.hk, 2, nt + mt * ratio); break;
+    default: out->grid[0] = persistent(grid1d(s.hk, 2, nt + mt * ratio)); break;
   }
   out->backend_index = be;
   out->head_dim = s.d;

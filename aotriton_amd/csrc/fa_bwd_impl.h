@@ -1126,22 +1126,29 @@ void bwd_fused_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   const int group = a.hq / a.hk;
   const int items = a.num_n_tiles + a.num_m_tiles * group;
-  const int xcd = blockIdx.x % kNumXcd, li = blockIdx.x / kNumXcd;
+  // persistent workgroups with the walk of the split kernels (one workgroup per item with a bias
+  // or at D = 256, where the loop runs once)
+  const int xcd = blockIdx.x % kNumXcd, p = blockIdx.x / kNumXcd, workers = gridDim.x / kNumXcd;
   const int per_group = a.zh_group * items;
-  const int gi = li / per_group, gr = li % per_group;
-  const int zl = gi * a.zh_group + gr % a.zh_group;
-  const int zh = xcd * a.zh_per_xcd + zl;
-  if (zl >= a.zh_per_xcd || zh >= a.num_zh) return;
-  int z, hk;
-  split_zh(zh, a.num_zh / a.hk, 1, z, hk);
-  const int item = gr / a.zh_group;
-  if (item < a.num_n_tiles) {
-    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true, kPad>(a, hk, item, z, smem_raw);
-  } else {
-    const int t = item - a.num_n_tiles;
-    const int h = hk * group + t / a.num_m_tiles;
-    const int mt = a.num_m_tiles - 1 - t % a.num_m_tiles;
-    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true, kPad>(a, h, mt, z, smem_raw);
+  for (int r = 0; D >= 256 ? r < 1 : r * workers < a.items_per_xcd; ++r) {
+    const int li = r * workers + ((r & 1) ? workers - 1 - p : p);
+    if (li >= a.items_per_xcd) continue;
+    const int gi = li / per_group, gr = li % per_group;
+    const int zl = gi * a.zh_group + gr % a.zh_group;
+    const int zh = xcd * a.zh_per_xcd + zl;
+    if (zl >= a.zh_per_xcd || zh >= a.num_zh) continue;
+    int z, hk;
+    split_zh(zh, a.num_zh / a.hk, 1, z, hk);
+    const int item = gr / a.zh_group;
+    if (item < a.num_n_tiles) {
+      dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, true, kPad>(a, hk, item, z, smem_raw);
+    } else {
+      const int t = item - a.num_n_tiles;
+      const int h = hk * group + t / a.num_m_tiles;
+      const int mt = a.num_m_tiles - 1 - t % a.num_m_tiles;
+      dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true, kPad>(a, h, mt, z, smem_raw);
+    }
+    __syncthreads();     // the next item reuses the LDS stages
   }
 }
 
@@ -1240,7 +1247,8 @@ hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dr
   a.zh_per_xcd = (a.num_zh + kNumXcd - 1) / kNumXcd;
   a.zh_group = 2;
   const int items = a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk);
-  dim3 grid((unsigned)(kNumXcd * ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * items));
+  a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * items;
+  dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
 #define FA_CALL(W, B, P) launch_with_lds<bwd_fused_kernel<T, D, NW, BM, BN, W, B, P, kPad>>(grid, NW * 64, smem, stream, a)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL

@@ -104,25 +104,6 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   char* rowbuf = smem_raw + SM::ROWS_OFF + wave * 32 * SM::ROW_STR;
   const int wrows = si.seqlen_q - q0 - wave * 32 < 32 ? si.seqlen_q - q0 - wave * 32 : 32;   // may be <= 0
   const int rq = lane / LPRQ, cq = lane % LPRQ;
-  op_t qreg[KS];
-  {
-    const T* qw = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
-                  (int64_t)(si.q_start + q0 + wave * 32) * a.sq.s;
-    const auto qrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qw), 0,
-                                                       wrows > 0 ? ((wrows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
-    const int qvoff = cq * 8 < d_qk ? rq * (int)a.sq.s * 2 + cq * 16 : kVoffOutOfRange;
-    op_t qin[32 / RPQ];
-#pragma unroll
-    for (int i = 0; i < 32 / RPQ; ++i)
-      qin[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(qrs, qvoff, i * RPQ * (int)a.sq.s * 2, 0));
-#pragma unroll
-    for (int i = 0; i < 32 / RPQ; ++i)
-      *reinterpret_cast<op_t*>(rowbuf + (i * RPQ + rq) * SM::ROW_STR + cq * 16) = qin[i];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qreg[ks] = *reinterpret_cast<const op_t*>(rowbuf + c * SM::ROW_STR + (16 * ks + 8 * hi) * 2);
-  }
-
   const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
                    (int64_t)hk * a.sk.h + (int64_t)si.k_start * a.sk.s;
   const T* vbase = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z +
@@ -175,6 +156,30 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
       vreg[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(vrs, vvoff, i * vsoff, 0));
     kt += k_step; vt += v_step; rows_left -= BN;
   };
+
+  // the first K/V tile is requested before the Q rows are waited for: both fetches are in flight
+  // together
+  load_next_tile();
+
+  op_t qreg[KS];
+  {
+    const T* qw = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
+                  (int64_t)(si.q_start + q0 + wave * 32) * a.sq.s;
+    const auto qrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qw), 0,
+                                                       wrows > 0 ? ((wrows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
+    const int qvoff = cq * 8 < d_qk ? rq * (int)a.sq.s * 2 + cq * 16 : kVoffOutOfRange;
+    op_t qin[32 / RPQ];
+#pragma unroll
+    for (int i = 0; i < 32 / RPQ; ++i)
+      qin[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(qrs, qvoff, i * RPQ * (int)a.sq.s * 2, 0));
+#pragma unroll
+    for (int i = 0; i < 32 / RPQ; ++i)
+      *reinterpret_cast<op_t*>(rowbuf + (i * RPQ + rq) * SM::ROW_STR + cq * 16) = qin[i];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qreg[ks] = *reinterpret_cast<const op_t*>(rowbuf + c * SM::ROW_STR + (16 * ks + 8 * hi) * 2);
+  }
+
 
   auto store_tile = [&](int stage) {
     T* ks = Ks + stage * SM::K_ELEMS + ldsk0;
@@ -442,7 +447,6 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   };
 
   // ---- main loop: LDS double buffer, one barrier per tile ---------------------
-  load_next_tile();
   store_tile(0);
   __syncthreads();
   for (int j = br.lo; j <= br.hi; ++j) {
