@@ -407,7 +407,7 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
   if (e != FA_SUCCESS) return e;
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
-  const fa::TileShape t = valu ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(s.d);
+  const fa::TileShape t = valu ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(params->Q.dtype, s.d, s.windowed);
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
   if (valu) {
@@ -444,7 +444,7 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
   if (valu && kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
   const fa::TileShape t = valu ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
-                               : fa::bwd_tile_shape(s.d, kernel_slot);
+                               : fa::bwd_tile_shape(params->Q.dtype, s.d, s.windowed, kernel_slot);
   const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
@@ -529,7 +529,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
   a.atomic_counter = static_cast<int32_t*>(p->persistent_atomic_counter.ptr);
   a.num_cu = dev->num_cu;
 
-  const fa::TileShape t = (p->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256) ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(s.d);
+  const fa::TileShape t = (p->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256) ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(p->Q.dtype, s.d, s.windowed);
   FA_LOG(4, "attn_fwd: D=%d BLOCK_M=%d BLOCK_N=%d waves=%d lds=%d windowed=%d bias=%d dropout=%d nseq=%d",
          s.d, t.block_m, t.block_n, t.num_waves, t.lds_bytes, (int)s.windowed, (int)s.bias,
          (int)s.dropout, s.num_seqlens);

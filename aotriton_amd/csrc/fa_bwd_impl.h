@@ -82,10 +82,16 @@ struct DqSmem {     // per stage: K, V (swizzled)
   static constexpr int BYTES = STAGES * STAGE_BYTES;
 };
 
-template <int D> struct BwdTile;   // NW waves; dK/dV: BN = 32*NW keys x BM queries; dQ: BM = 32*NW queries x BN keys
-template <> struct BwdTile<64>  { static constexpr int NW = 4, DKDV_BM = 128, DQ_BN = 128; };
-template <> struct BwdTile<128> { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
-template <> struct BwdTile<256> { static constexpr int NW = 4, DKDV_BM = 32, DQ_BN = 32; };
+// Tile table of the backward kernels, keyed on (element type, head dim, causal / windowed).  NW
+// waves; dK/dV: 32*NW keys per workgroup, DKDV_BM queries per step; dQ: 32*NW queries per
+// workgroup, DQ_BN keys per step.  The reference keeps separate tuned tiles for causal and
+// non-causal shapes (its database has 64x16 / 64x32 for dK/dV and 64x64 / 64x32 for dQ at the
+// headline shape); here the same tile wins on both sides of every key (same-box A/B at D = 128,
+// bf16: 32-query / 32-key steps lose 6 % causal and 7-10 % non-causal on each kernel).
+template <typename T, int D, bool kWindowed> struct BwdTile;
+template <typename T, bool kWindowed> struct BwdTile<T, 64, kWindowed>  { static constexpr int NW = 4, DKDV_BM = 128, DQ_BN = 128; };
+template <typename T, bool kWindowed> struct BwdTile<T, 128, kWindowed> { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
+template <typename T, bool kWindowed> struct BwdTile<T, 256, kWindowed> { static constexpr int NW = 4, DKDV_BM = 32, DQ_BN = 32; };
 
 // ---------------------------------------------------------------------------
 // dK / dV work item
@@ -1206,9 +1212,10 @@ hipError_t launch_bwd_preprocess(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <typename T, int D, bool kPad>
-hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
-  constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = NW * 32;
+template <typename T, int D, bool kPad, bool W, bool B, bool P>
+hipError_t launch_dkdv_variant(const BwdArgs& a0, hipStream_t stream) {
+  using Tile = BwdTile<T, D, W>;
+  constexpr int NW = Tile::NW, BM = Tile::DKDV_BM, BN = NW * 32;
   BwdArgs a = a0;
   a.num_n_tiles = (a.seq.max_seqlen_k + BN - 1) / BN;
   a.num_zh = bwd_nseq(a) * a.hk;
@@ -1216,14 +1223,20 @@ hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dro
   a.zh_group = 2;
   a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles;
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
-#define FA_CALL(W, B, P) launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>>(grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a)
+  return launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>>(grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a);
+}
+
+template <typename T, int D, bool kPad>
+hipError_t launch_bwd_dkdv(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+#define FA_CALL(W, B, P) launch_dkdv_variant<T, D, kPad, W, B, P>(a0, stream)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
 
-template <typename T, int D, bool kPad>
-hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
-  constexpr int NW = BwdTile<D>::NW, BN = BwdTile<D>::DQ_BN, BM = NW * 32;
+template <typename T, int D, bool kPad, bool W, bool B, bool P>
+hipError_t launch_dq_variant(const BwdArgs& a0, hipStream_t stream) {
+  using Tile = BwdTile<T, D, W>;
+  constexpr int NW = Tile::NW, BN = Tile::DQ_BN, BM = NW * 32;
   BwdArgs a = a0;
   a.num_m_tiles = (a.seq.max_seqlen_q + BM - 1) / BM;
   a.num_zh = bwd_nseq(a) * a.hq;
@@ -1231,14 +1244,20 @@ hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropo
   a.zh_group = a.hq / a.hk > 2 ? (a.hq / a.hk > 8 ? 8 : a.hq / a.hk) : 2;
   a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_m_tiles;
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
-#define FA_CALL(W, B, P) launch_with_lds<bwd_dq_kernel<T, D, NW, BN, W, B, P, kPad>>(grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a)
+  return launch_with_lds<bwd_dq_kernel<T, D, NW, BN, W, B, P, kPad>>(grid, NW * 64, DqSmem<D, BN>::BYTES, stream, a);
+}
+
+template <typename T, int D, bool kPad>
+hipError_t launch_bwd_dq(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+#define FA_CALL(W, B, P) launch_dq_variant<T, D, kPad, W, B, P>(a0, stream)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
 
-template <typename T, int D, bool kPad>
-hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
-  constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = BwdTile<D>::DQ_BN;
+template <typename T, int D, bool kPad, bool W, bool B, bool P>
+hipError_t launch_fused_variant(const BwdArgs& a0, hipStream_t stream) {
+  using Tile = BwdTile<T, D, W>;
+  constexpr int NW = Tile::NW, BM = Tile::DKDV_BM, BN = Tile::DQ_BN;
   constexpr int smem = DkDvSmem<D, BM>::BYTES > DqSmem<D, BN>::BYTES ? DkDvSmem<D, BM>::BYTES : DqSmem<D, BN>::BYTES;
   BwdArgs a = a0;
   a.num_n_tiles = (a.seq.max_seqlen_k + NW * 32 - 1) / (NW * 32);
@@ -1249,13 +1268,19 @@ hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dr
   const int items = a.num_n_tiles + a.num_m_tiles * (a.hq / a.hk);
   a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * items;
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
-#define FA_CALL(W, B, P) launch_with_lds<bwd_fused_kernel<T, D, NW, BM, BN, W, B, P, kPad>>(grid, NW * 64, smem, stream, a)
+  return launch_with_lds<bwd_fused_kernel<T, D, NW, BM, BN, W, B, P, kPad>>(grid, NW * 64, smem, stream, a);
+}
+
+template <typename T, int D, bool kPad>
+hipError_t launch_bwd_fused(const BwdArgs& a0, bool windowed, bool bias, bool dropout, hipStream_t stream) {
+#define FA_CALL(W, B, P) launch_fused_variant<T, D, kPad, W, B, P>(a0, stream)
   FA_BWD_SWITCH(FA_CALL)
 #undef FA_CALL
 }
 
-template <int D> TileShape bwd_shape(int slot) {
-  constexpr int NW = BwdTile<D>::NW, BM = BwdTile<D>::DKDV_BM, BN = BwdTile<D>::DQ_BN;
+template <typename T, int D, bool kWindowed> TileShape bwd_shape(int slot) {
+  using Tile = BwdTile<T, D, kWindowed>;
+  constexpr int NW = Tile::NW, BM = Tile::DKDV_BM, BN = Tile::DQ_BN;
   constexpr int s1 = DkDvSmem<D, BM>::BYTES, s2 = DqSmem<D, BN>::BYTES;
   switch (slot) {
     case 0: return TileShape{256 / (D / 8), 0, 4, 0};

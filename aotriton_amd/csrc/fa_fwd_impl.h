@@ -56,7 +56,13 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   T* Vs = Ks + SM::STAGES * SM::K_ELEMS;
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
+  // At D = 256 (one wave per SIMD, accumulators in AGPRs) the wave index is taken as a scalar:
+  // the branches on it are then uniform for the compiler too, and it keeps the copies of the 128
+  // accumulator registers that the rarely taken full softmax step needs out of the common path
+  // (they doubled the vector instructions per tile of the causal kernel: 737 -> 895 TFLOP/s at
+  // S = 16384).  At D <= 128 there are no AGPRs and the plain form measures 0-4 % faster.
+  const int wave = D >= 256 ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;
+  const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
   // columns of Q/K and of V/Out: <= D, multiples of 8; constants unless a head dim is rounded up
   const int d_qk = kPad ? a.head_dim : D, d_v = kPad ? a.head_dim_v : D;
 
@@ -536,15 +542,25 @@ void fwd_kernel(const FwdArgs a) {
   }
 }
 
-// Tile table: one entry per head dim.
-template <int D> struct FwdTile;
-template <> struct FwdTile<64>  { static constexpr int NW = 8, BN = 128; };
-template <> struct FwdTile<128> { static constexpr int NW = 8, BN = 64; };
-template <> struct FwdTile<256> { static constexpr int NW = 4, BN = 32; };
+// Tile table of the forward kernel, keyed on (element type, head dim, causal / windowed): NW waves
+// of 32 queries each, BN keys per K/V tile.  This is what replaces the reference's tuning
+// database for attn_fwd (modules/flash/aot/attn_fwd.py:69-80 lists its candidate tiles, which
+// differ between causal and non-causal).  Here the measured best tile is the same on both sides
+// of every key; the alternatives that lost are noted per entry (same-box A/B, bf16, B*H*D = 16384,
+// S = 4096 and 16384).
+template <typename T, int D, bool kWindowed> struct FwdTile;
+// D = 64: 128-key tiles; 64-key tiles lose 2 % causal and 6 % non-causal at S = 4096.
+template <typename T, bool kWindowed> struct FwdTile<T, 64, kWindowed>  { static constexpr int NW = 8, BN = 128; };
+// D = 128: 64-key tiles; 32-key tiles (finer skipping on the causal diagonal, twice the barriers)
+// lose 6-7 % causal and 5 % non-causal.  128-key tiles do not fit the LDS next to the row areas.
+template <typename T, bool kWindowed> struct FwdTile<T, 128, kWindowed> { static constexpr int NW = 8, BN = 64; };
+// D = 256: one wave per SIMD (the accumulators of 32 rows take 128 registers), 32-key tiles; 64-key
+// tiles spill.
+template <typename T, bool kWindowed> struct FwdTile<T, 256, kWindowed> { static constexpr int NW = 4, BN = 32; };
 
 template <typename T, int D, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
-  constexpr int NW = FwdTile<D>::NW, BN = FwdTile<D>::BN;
+  constexpr int NW = FwdTile<T, D, kWindowed>::NW, BN = FwdTile<T, D, kWindowed>::BN;
   auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>;
   constexpr int smem = FwdSmem<D, BN, NW>::BYTES;
   if (grid.x == 0) return hipSuccess;      // no batch, no head or no query row: nothing to write
@@ -561,7 +577,7 @@ hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
 // columns are masked.
 template <typename T, int D, bool kPad>
 hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t stream) {
-  constexpr int BM = FwdTile<D>::NW * 32;
+  const int BM = (windowed ? FwdTile<T, D, true>::NW : FwdTile<T, D, false>::NW) * 32;
   const int nseq = a.seq.num_seqlens != 0 ? (a.seq.num_seqlens < 0 ? -a.seq.num_seqlens : a.seq.num_seqlens)
                                           : a.batch;
   FwdArgs b = a;

@@ -17,7 +17,8 @@ hipError_t run_fwd_d256(int dtype, const FwdArgs& a, bool windowed, bool bias, b
 hipError_t run_fwd_d64_padded(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_fwd_d128_padded(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_fwd_d256_padded(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
-TileShape fwd_tile_shape(int head_dim);
+// tile table lookups: (element type, head dim, causal / windowed)
+TileShape fwd_tile_shape(int dtype, int head_dim, bool windowed);
 
 hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s);
 // register-only MFMA loop: the rate the matrix pipe sustains (benchmark aid)
@@ -28,7 +29,7 @@ hipError_t run_bwd_preprocess(int dtype, int head_dim, const BwdArgs& a, hipStre
 hipError_t run_bwd_dkdv(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_bwd_dq(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_bwd_fused(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
-TileShape bwd_tile_shape(int head_dim, int kernel_slot);
+TileShape bwd_tile_shape(int dtype, int head_dim, bool windowed, int kernel_slot);
 
 // Vector-ALU kernels (no MFMA): fp32 tensors at any head dim, every type at head dim 512.
 // head_dim is the compiled one (64, 128, 256, 512).  kernel_slot of the backward: 0 delta,

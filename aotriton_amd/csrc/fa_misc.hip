@@ -84,6 +84,5 @@ hipError_t run_mfma_rate(bool random_operands, int grid, int iters, float* out, 
   return hipGetLastError();
 }
 
-TileShape fwd_tile_shape(int head_dim);
 
 }  // namespace fa

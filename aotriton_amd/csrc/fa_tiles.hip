@@ -1,28 +1,39 @@
-// Compile-time tile/occupancy table, reported through fa_query_*_config.
+// Compile-time tile/occupancy table keyed on (element type, head dim, causal / windowed), reported
+// through fa_query_*_config.
 #include "fa_fwd_impl.h"
 #include "fa_bwd_impl.h"
 #include "fa_kernels.h"
 
 namespace fa {
 
-template <int D> static TileShape fwd_shape() {
-  return TileShape{FwdTile<D>::NW * 32, FwdTile<D>::BN, FwdTile<D>::NW, FwdSmem<D, FwdTile<D>::BN, FwdTile<D>::NW>::BYTES};
+template <typename T, int D, bool W> static TileShape fwd_shape() {
+  using Tile = FwdTile<T, D, W>;
+  return TileShape{Tile::NW * 32, Tile::BN, Tile::NW, FwdSmem<D, Tile::BN, Tile::NW>::BYTES};
 }
 
-TileShape fwd_tile_shape(int head_dim) {
+template <typename T> static TileShape fwd_shape_of(int head_dim, bool windowed) {
   switch (head_dim) {
-    case 64: return fwd_shape<64>();
-    case 128: return fwd_shape<128>();
-    default: return fwd_shape<256>();
+    case 64: return windowed ? fwd_shape<T, 64, true>() : fwd_shape<T, 64, false>();
+    case 128: return windowed ? fwd_shape<T, 128, true>() : fwd_shape<T, 128, false>();
+    default: return windowed ? fwd_shape<T, 256, true>() : fwd_shape<T, 256, false>();
   }
 }
 
-TileShape bwd_tile_shape(int head_dim, int kernel_slot) {
+TileShape fwd_tile_shape(int dtype, int head_dim, bool windowed) {
+  return dtype == kDtypeBF16 ? fwd_shape_of<bf16_t>(head_dim, windowed) : fwd_shape_of<f16_t>(head_dim, windowed);
+}
+
+template <typename T> static TileShape bwd_shape_of(int head_dim, bool windowed, int slot) {
   switch (head_dim) {
-    case 64: return bwd_shape<64>(kernel_slot);
-    case 128: return bwd_shape<128>(kernel_slot);
-    default: return bwd_shape<256>(kernel_slot);
+    case 64: return windowed ? bwd_shape<T, 64, true>(slot) : bwd_shape<T, 64, false>(slot);
+    case 128: return windowed ? bwd_shape<T, 128, true>(slot) : bwd_shape<T, 128, false>(slot);
+    default: return windowed ? bwd_shape<T, 256, true>(slot) : bwd_shape<T, 256, false>(slot);
   }
+}
+
+TileShape bwd_tile_shape(int dtype, int head_dim, bool windowed, int kernel_slot) {
+  return dtype == kDtypeBF16 ? bwd_shape_of<bf16_t>(head_dim, windowed, kernel_slot)
+                             : bwd_shape_of<f16_t>(head_dim, windowed, kernel_slot);
 }
 
 }  // namespace fa

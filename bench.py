@@ -92,6 +92,9 @@ def main():
     ap.add_argument('--traffic-probe', action='store_true',
                     help='also run one elementwise kernel of known HBM traffic (256 MiB read + 256 MiB '
                          'written) so that FETCH_SIZE / WRITE_SIZE counters can be scaled')
+    ap.add_argument('--tile-entry', default=None, metavar='D,causal,dtype',
+                    help='run the forward, dK/dV and dQ kernels of one tile-table entry a few times and print their '
+                         'times (for profiler runs), e.g. 64,1,bf16: B = 4, H = 4096 / D, S = 4096')
     ap.add_argument('--mfma-peak', action='store_true',
                     help='only measure what the matrix pipe sustains (register-only MFMA loop, constant '
                          'and random operands) and print that as one JSON line')
@@ -142,6 +145,43 @@ def main():
         t = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
         q = lambda p: t[min(n - 1, int(p * n))]
         return {'median': q(0.5), 'p20': q(0.2), 'p80': q(0.8), 'mean': sum(t) / n, 'reps': n}
+
+    if args.tile_entry:
+        d_s, c_s, t_s = args.tile_entry.split(',')
+        D, causal = int(d_s), bool(int(c_s))
+        dtype = {'bf16': torch.bfloat16, 'fp16': torch.float16}[t_s]
+        B, S = 4, 4096
+        H = 4096 // D
+        g = torch.Generator(device=dev).manual_seed(1234)
+        rn = lambda: torch.randn(B, H, S, D, device=dev, dtype=torch.float32, generator=g).to(dtype)
+        q, k, v, do = rn(), rn(), rn(), rn()
+        o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+        L = torch.empty(B * H, S, device=dev, dtype=torch.float32)
+        delta = torch.empty_like(L)
+        null = torch.empty([0], device=dev, dtype=torch.uint64)
+        atomic = torch.zeros([1], device=dev, dtype=torch.int32)
+        sm = 1.0 / math.sqrt(D)
+        bp = attn_bwd_params()
+        flash._fill_bwd(bp, q, k, v, None, sm, o, do, dq, dk, dv, None, None, L, delta, 0.0, null, null, 0, causal)
+        fns = {'fwd': lambda: flash.attn_fwd(q, k, v, None, sm, L, o, 0.0, null, null, 0, null, null, None, causal, atomic),
+               'bwd_preprocess': lambda: attn_bwd_kernel(bp, attn_bwd_params.kVersion, flash._stream(), 0),
+               'bwd_dkdv': lambda: attn_bwd_kernel(bp, attn_bwd_params.kVersion, flash._stream(), 1),
+               'bwd_dq': lambda: attn_bwd_kernel(bp, attn_bwd_params.kVersion, flash._stream(), 2)}
+        res = {}
+        for name, fn in fns.items():
+            assert fn() == ok
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(5):
+                fn()
+            e1.record()
+            e1.synchronize()
+            res[name + '_ms'] = e0.elapsed_time(e1) / 5
+        gemm = 2.0 * B * H * S * S * D * (0.5 if causal else 1.0)
+        print(json.dumps({'tile_entry': args.tile_entry, 'B': B, 'H': H, 'S': S, 'D': D, 'causal': causal,
+                          'flop_per_gemm': gemm, **res}))
+        return
 
     if args.mfma_peak:
         grid, iters = 512, 40000
