@@ -794,6 +794,18 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   } else {
     d_row = a.delta[lo];
   }
+  // The resident Q / dO operands live in accumulation registers: an MFMA takes its B operand
+  // from there directly.  Left to itself the register allocator parks them there as well (the
+  // kernel needs more than 256 registers) but copies each one back before every use: 32-44
+  // copies per key tile at D = 128, a quarter of the loop's vector instructions.  Not at
+  // D = 256, where the allocation gets worse with the constraint.
+  if constexpr (D <= 128) {
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      asm volatile("" : "+a"(qreg[k]));
+      asm volatile("" : "+a"(doreg[k]));
+    }
+  }
 
   // Without dropout (the mask and the scale come between dP and the subtraction) dP starts at
   // -delta.  Not in the dQ kernel at D = 64: with 128-key tiles its register allocation gets
