@@ -20,6 +20,7 @@
 #include <type_traits>
 
 #include "fa_device.h"
+#include "fa_fwd_pipe.h"
 
 namespace fa {
 
@@ -509,9 +510,11 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 // interleaved, and the workgroups of the XCD take them in serpentine order (worker p
 // takes p, 2P-1-p, 2P+p, ...), which pairs heavy with light tiles.  A workgroup
 // goes from one tile to the next without a relaunch.
-template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kPad>
+// QB = 0: fwd_item, NW waves of 32 rows.  QB > 0: fwd_item_pipe, 4 waves of 32 * QB rows, one wave
+// per SIMD.
+template <typename T, int D, int NW, int BN, int QB, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
-__attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1, D <= 128 ? 2 : 1)))
+__attribute__((amdgpu_waves_per_eu(D <= 128 && QB == 0 ? 2 : 1, D <= 128 && QB == 0 ? 2 : 1)))
 void fwd_kernel(const FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   if (kDropout && blockIdx.x == 0 && threadIdx.x == 0) {
@@ -538,7 +541,8 @@ void fwd_kernel(const FwdArgs a) {
     const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
     int z, h;
     split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
-    fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>(a, z, h, mt, smem_raw);
+    if constexpr (QB > 0) fwd_item_pipe<T, D, QB, BN, kWindowed, kBias, kDropout, kPad>(a, z, h, mt, smem_raw);
+    else fwd_item<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>(a, z, h, mt, smem_raw);
   }
 }
 
@@ -548,21 +552,32 @@ void fwd_kernel(const FwdArgs a) {
 // differ between causal and non-causal).  Here the measured best tile is the same on both sides
 // of every key; the alternatives that lost are noted per entry (same-box A/B, bf16, B*H*D = 16384,
 // S = 4096 and 16384).
+template <int D_, int NW_, int BN_, int QB_> struct FwdTileOf {
+  static constexpr int NW = NW_, BN = BN_, QB = QB_;
+  static constexpr int BM = NW * 32 * (QB > 0 ? QB : 1);
+  static constexpr int LDS = QB > 0 ? FwdPipeSmem<D_, BN, (QB > 0 ? QB : 1)>::BYTES : FwdSmem<D_, BN, NW>::BYTES;
+};
 template <typename T, int D, bool kWindowed> struct FwdTile;
 // D = 64: 128-key tiles; 64-key tiles lose 2 % causal and 6 % non-causal at S = 4096.
-template <typename T, bool kWindowed> struct FwdTile<T, 64, kWindowed>  { static constexpr int NW = 8, BN = 128; };
+template <typename T, bool kWindowed> struct FwdTile<T, 64, kWindowed> : FwdTileOf<64, 8, 128, 0> {};
 // D = 128: 64-key tiles; 32-key tiles (finer skipping on the causal diagonal, twice the barriers)
 // lose 6-7 % causal and 5 % non-causal.  128-key tiles do not fit the LDS next to the row areas.
-template <typename T, bool kWindowed> struct FwdTile<T, 128, kWindowed> { static constexpr int NW = 8, BN = 64; };
-// D = 256: one wave per SIMD (the accumulators of 32 rows take 128 registers), 32-key tiles; 64-key
-// tiles spill.
-template <typename T, bool kWindowed> struct FwdTile<T, 256, kWindowed> { static constexpr int NW = 4, BN = 32; };
+template <typename T, bool kWindowed> struct FwdTile<T, 128, kWindowed> : FwdTileOf<128, 8, 64, 0> {};
+// (The pipelined item with 64 rows per wave, FwdTileOf<128, 4, 64, 2>, halves the LDS operand traffic
+// per MFMA but measures 20 % slower than this one at S = 4096 and 16384: one wave per SIMD issues
+// its MFMAs, vector and LDS instructions one after the other, and two waves overlap better.)
+// D = 256: one wave per SIMD (the accumulators of 32 rows take 128 registers), 32-key tiles, the
+// software-pipelined item: level with fwd_item without bias and dropout (B2 H16 S8192 fp16: 903 vs
+// 875 TFLOP/s non-causal, 827 vs 835 causal), 15-25 % faster with them (bias: 644 vs 553, causal
+// 629 vs 510; bias + dropout + window 1024: 361 vs 333).
+template <typename T, bool kWindowed> struct FwdTile<T, 256, kWindowed> : FwdTileOf<256, 4, 32, 1> {};
 
 template <typename T, int D, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
-  constexpr int NW = FwdTile<T, D, kWindowed>::NW, BN = FwdTile<T, D, kWindowed>::BN;
-  auto kern = fwd_kernel<T, D, NW, BN, kWindowed, kBias, kDropout, kPad>;
-  constexpr int smem = FwdSmem<D, BN, NW>::BYTES;
+  using Tile = FwdTile<T, D, kWindowed>;
+  constexpr int NW = Tile::NW;
+  auto kern = fwd_kernel<T, D, NW, Tile::BN, Tile::QB, kWindowed, kBias, kDropout, kPad>;
+  constexpr int smem = Tile::LDS;
   if (grid.x == 0) return hipSuccess;      // no batch, no head or no query row: nothing to write
   if (smem > 64 * 1024) {
     static std::atomic<uint64_t> lds_set{0};
@@ -577,7 +592,7 @@ hipError_t launch_fwd_variant(const FwdArgs& a, dim3 grid, hipStream_t stream) {
 // columns are masked.
 template <typename T, int D, bool kPad>
 hipError_t launch_fwd(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t stream) {
-  const int BM = (windowed ? FwdTile<T, D, true>::NW : FwdTile<T, D, false>::NW) * 32;
+  const int BM = windowed ? FwdTile<T, D, true>::BM : FwdTile<T, D, false>::BM;
   const int nseq = a.seq.num_seqlens != 0 ? (a.seq.num_seqlens < 0 ? -a.seq.num_seqlens : a.seq.num_seqlens)
                                           : a.batch;
   FwdArgs b = a;

@@ -8,7 +8,7 @@ namespace fa {
 
 template <typename T, int D, bool W> static TileShape fwd_shape() {
   using Tile = FwdTile<T, D, W>;
-  return TileShape{Tile::NW * 32, Tile::BN, Tile::NW, FwdSmem<D, Tile::BN, Tile::NW>::BYTES};
+  return TileShape{Tile::BM, Tile::BN, Tile::NW, Tile::LDS};
 }
 
 template <typename T> static TileShape fwd_shape_of(int head_dim, bool windowed) {
