@@ -75,11 +75,13 @@ struct DkDvSmem {   // per stage: Q, dO (swizzled, one copy each); L, delta; bia
 };
 
 template <int D, int BN>
-struct DqSmem {     // per stage: K, V (swizzled)
+struct DqSmem {     // per stage: K, V (swizzled); then one bias / dB tile per wave (32 rows, +16 B per row)
   static constexpr int TILE_BYTES = BN * D * 2;
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES;
   static constexpr int STAGES = 2;
-  static constexpr int BYTES = STAGES * STAGE_BYTES;
+  static constexpr int BIAS_OFF = STAGES * STAGE_BYTES;
+  static constexpr int BIAS_ROW = BN * 2 + 16;
+  static constexpr int BYTES = BIAS_OFF + 4 * 32 * BIAS_ROW;
 };
 
 // Tile table of the backward kernels, keyed on (element type, head dim, causal / windowed).  NW
@@ -828,6 +830,28 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
                         (reinterpret_cast<uintptr_t>(a.bias) & 7) == 0;
   const bool db_vec = kBias && a.sdb_n == 1 && ((a.sdb_m | a.sdb_h | a.sdb_z) & 3) == 0 &&
                       (reinterpret_cast<uintptr_t>(a.db) & 7) == 0;
+  // Whole tiles of bias and dB travel as row-contiguous 16-byte pieces (consecutive lanes along a
+  // row: a wave-wide access touches 64 / (BN / 8) rows) and change to the one-row-per-lane layout
+  // of the MFMA results in a 32-row LDS area of the wave.  One 8-byte access per lane and 4 keys
+  // touches 32 cache lines for 16 bytes each, and the vector memory pipe's line rate then makes a
+  // bias cost more than all the MFMAs of the kernel (dQ with bias 4.4 ms against 1.6 ms without).
+  constexpr int BLPR = BN / 8;            // 16-byte pieces per tile row
+  constexpr int BRPI = 64 / BLPR;         // rows per wave-wide access
+  constexpr int BNI = 32 / BRPI;          // accesses per tile
+  char* bw = smem_raw + SM::BIAS_OFF + wave * 32 * SM::BIAS_ROW;
+  const int brow = lane / BLPR, bch = lane % BLPR;
+  const bool bias_co = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 7) == 0 &&
+                       (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0;
+  const bool db_co = kBias && a.db != nullptr && a.sdb_n == 1 && ((a.sdb_m | a.sdb_h | a.sdb_z) & 7) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.db) & 15) == 0;
+  // an item's tiles take the vector code when the bias can be read as vectors and dB (if wanted)
+  // written through the LDS area
+  const bool want_db = kBias && a.db != nullptr;
+  const bool item_fast = !kBias || (bias_vec && (!want_db || (db_co && db_vec)));
+  const T* bias_head = kBias ? reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
+                                   (int64_t)h * a.sb_h : nullptr;
+  T* db_head = kBias && a.db != nullptr ? reinterpret_cast<T*>(a.db) + (int64_t)si.batch_index * a.sdb_z +
+                                              (int64_t)h * a.sdb_h : nullptr;
   DropoutState dst{};
   if (kDropout) dst = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
 
@@ -888,8 +912,13 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = vch[i - CH];
   };
 
-  auto compute = [&](auto masked_tag, int j, int stage, bool live) {
+  // kFast (bias only): the tile lies inside the key range and bias and dB can travel as vectors; the
+  // element code then has no run-time branch.  Other tiles of a bias run take the general code, in a
+  // loop of their own: one loop body holding both would branch around every element and move the
+  // accumulators between the two copies of its MFMAs.
+  auto compute = [&](auto masked_tag, auto fast_tag, int j, int stage, bool live) {
     constexpr bool masked = decltype(masked_tag)::value;
+    constexpr bool kFast = decltype(fast_tag)::value;
     constexpr int G1 = KS * MB, G4 = TS * DB;
     const char* Kb = smem_raw + stage * SM::STAGE_BYTES;
     const char* Vb = Kb + SM::TILE_BYTES;
@@ -902,8 +931,25 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     op_t xa[kAhead + 1][MB];
     op_t sb[TS];
     uint32_t keep[kDropout ? 4 * MB : 1];
-    q4_t bias4[2];
-    const bool tile_vec = bias_vec && (j + 1) * BN <= si.seqlen_k;   // the whole tile is inside the row
+    const bool tile_vec = kFast;
+    // the tile's bias, requested before the S MFMAs and used behind the dP MFMAs: with one wave per
+    // SIMD a load that is used where it is issued costs its whole latency
+    q4_t bias4[kBias ? 4 * MB : 1];
+    const bool tile_co = kFast && bias_co;                     // bias through the wave's LDS area
+    const bool tile_dbco = kFast && want_db;                   // dB through it
+    op_t bco[kBias ? BNI : 1];
+    if (kBias && tile_co) {
+#pragma unroll
+      for (int i = 0; i < BNI; ++i) {
+        int m = q0 + wave * 32 + brow + BRPI * i;
+        m = m < si.seqlen_q ? m : si.seqlen_q - 1;
+        bco[i] = *reinterpret_cast<const op_t*>(bias_head + (int64_t)m * a.sb_m + j * BN + bch * 8);
+      }
+    } else if (kBias && tile_vec) {
+#pragma unroll
+      for (int q = 0; q < 4 * MB; ++q)
+        bias4[q] = *reinterpret_cast<const q4_t*>(bptr + j * BN + 32 * (q / 4) + 8 * (q % 4) + 4 * hi);
+    }
 
     // ---- S^T = K Q^T -------------------------------------------------------------
 #pragma unroll
@@ -939,6 +985,15 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     for (int k = 0; k < kAhead; ++k)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Vb, row_a, k, mb);
+    if (kBias && tile_co) {
+      // (the wave's LDS operations run in order: the previous tile's dB pieces have left the area)
+#pragma unroll
+      for (int i = 0; i < BNI; ++i)
+        *reinterpret_cast<op_t*>(bw + (brow + BRPI * i) * SM::BIAS_ROW + bch * 16) = bco[i];
+#pragma unroll
+      for (int q = 0; q < 4 * MB; ++q)
+        bias4[q] = *reinterpret_cast<const q4_t*>(bw + c * SM::BIAS_ROW + (32 * (q / 4) + 8 * (q % 4) + 4 * hi) * 2);
+    }
 
     // element E = 16*mb + i of the tile: p, kept in s
     auto p_el = [&](int E) {
@@ -947,9 +1002,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       float x;
       if (kBias) {
         float bv;
-        if (tile_vec) {
-          if (r == 0) bias4[(E / 4) & 1] = *reinterpret_cast<const q4_t*>(bptr + n);
-          bv = (float)bias4[(E / 4) & 1][r];
+        if constexpr (kFast) {
+          bv = (float)bias4[E / 4][r];
         } else {
           const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
           bv = (float)bptr[(int64_t)nn * a.sb_n];
@@ -974,17 +1028,16 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       // where the dP accumulators start at -delta, dP - delta leaves the matrix pipe
       const float dsv = kFoldDelta ? s[mb][i] * dpv : s[mb][i] * (dpv - d_row);
       dp[mb][i] = dsv;
-      if (kBias && dbptr != nullptr && row_ok) {                                 // bwd_inner_dq.py:200-204
-        if (tile_vec && db_vec) {
-          if (r == 3) {
-            q4_t d4v;
+      if constexpr (kBias && kFast) {                                            // bwd_inner_dq.py:200-204
+        // (rows past the sequence write their part of the area too; it is never stored)
+        if (r == 3 && tile_dbco) {
+          q4_t d4v;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) d4v[q] = Tr::cvt(dp[mb][i - 3 + q]);
-            *reinterpret_cast<q4_t*>(dbptr + n - 3) = d4v;
-          }
-        } else if (n < si.seqlen_k) {
-          dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);
+          for (int q = 0; q < 4; ++q) d4v[q] = Tr::cvt(dp[mb][i - 3 + q]);
+          *reinterpret_cast<q4_t*>(bw + c * SM::BIAS_ROW + (32 * mb + 8 * g + 4 * hi) * 2) = d4v;
         }
+      } else if (kBias && dbptr != nullptr && row_ok) {
+        if (n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);
       }
       if (E & 1) {   // ds cast to K's dtype, pair by pair
         sb[E / 8][E % 8 - 1] = Tr::cvt(dp[mb][i - 1]);
@@ -1040,6 +1093,15 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    if (kBias && tile_dbco) {
+      // the wave's dB tile leaves as whole 16-byte pieces of its rows
+#pragma unroll
+      for (int i = 0; i < BNI; ++i) {
+        const int m = q0 + wave * 32 + brow + BRPI * i;
+        const op_t x = *reinterpret_cast<const op_t*>(bw + (brow + BRPI * i) * SM::BIAS_ROW + bch * 16);
+        if (m < si.seqlen_q) *reinterpret_cast<op_t*>(db_head + (int64_t)m * a.sdb_m + j * BN + bch * 8) = x;
+      }
+    }
   };
 
   fetch_begin(true);
@@ -1051,17 +1113,28 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   // K tiles come as [masked | full | masked]; one straight-line loop per run
   {
     int j = br.lo;
-    auto step = [&](auto masked_tag) {
+    auto step = [&](auto masked_tag, auto fast_tag) {
       const int stage = (j - br.lo) & 1;
-      compute(masked_tag, j, stage, j < br.hi);
+      compute(masked_tag, fast_tag, j, stage, j < br.hi);
       __syncthreads();
       ++j;
     };
     const int full_lo = br.fb_lo <= br.fb_hi ? br.fb_lo : br.hi + 1;
     const int full_hi = br.fb_lo <= br.fb_hi ? br.fb_hi : br.hi;
-    while (j < full_lo) step(std::true_type{});
-    while (j <= full_hi) step(std::false_type{});
-    while (j <= br.hi) step(std::true_type{});
+    // last tile that lies inside the key range (the vector code of a bias run ends there)
+    const int j_in = item_fast ? si.seqlen_k / BN - 1 : br.lo - 1;
+    auto run = [&](auto masked_tag, int upto) {
+      if constexpr (kBias) {
+        const int fast_to = upto < j_in ? upto : j_in;
+        while (j <= fast_to) step(masked_tag, std::true_type{});
+        while (j <= upto) step(masked_tag, std::false_type{});
+      } else {
+        while (j <= upto) step(masked_tag, std::true_type{});
+      }
+    };
+    run(std::true_type{}, full_lo - 1);
+    run(std::false_type{}, full_hi);
+    run(std::true_type{}, br.hi);
   }
 
   if (row_ok) {
