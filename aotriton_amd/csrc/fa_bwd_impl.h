@@ -235,6 +235,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   const T* bb_tile = nullptr;     // bias tile being fetched, its valid rows
   int b_rows = 0;
   const int b_cols = si.seqlen_k - n0 < BN ? si.seqlen_k - n0 : BN;      // valid keys of this item
+  const bool bias_plain = bias_lds && (b_cols & 7) == 0;                 // no piece straddles the end of a row
   // (g, e) = (q-head inside the GQA group, Q tile inside the range) of the tile to fetch;
   // called for consecutive tiles only; `live` false: nothing is fetched
   auto fetch_begin = [&](bool live, int g, int e) {
@@ -274,7 +275,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   auto fetch_piece = [&](int i) {        // Q pieces first, then dO (and O), then bias
     if (i >= 2 * CH) {
       const int k = i - 2 * CH;
-      if (bias_lds) {
+      if (bias_plain) {
+        // (the usual case behind one scalar branch: the two below test per lane)
+        bch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_voff, k * b_soff, 0));
+      } else if (bias_lds) {
         bch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_voff, k * b_soff, 0));
         // The descriptor ends at the last valid element of the tile's last row.  When that is
         // not at a 16-byte boundary the piece that straddles the end loses its valid elements
@@ -352,8 +356,11 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const char* dOb = sp + SM::TILE_BYTES;
     const float* Ls = reinterpret_cast<const float*>(sp + 2 * SM::TILE_BYTES);
     const float* Ds = Ls + BM;
-    // this lane's key column of the staged bias tile
-    const T* Bs = reinterpret_cast<const T*>(sp + 2 * SM::TILE_BYTES + 2 * BM * 4) + wave * 32 + c;
+    // The staged bias tile is row-major (queries x keys) and a lane needs its key's column: a
+    // transposing read hands each lane four consecutive queries of its key (lane i of a group of
+    // 16 gets, in slot j, element i % 4 of the 8 bytes addressed by lane 4 j + i / 4).
+    const char* Bt = sp + 2 * SM::TILE_BYTES + 2 * BM * 4 + (4 * hi + (lane & 15) / 4) * SM::BIAS_STR +
+                     (wave * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
     f32x16 s[MB], dp[MB];
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -427,6 +434,12 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     }
     // row statistics of the tile's queries and the first dO operands
     l4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ls, 0));
+    typename Tr::q4_t bias4[kBias ? 4 * MB : 1];
+    if (kBias) {
+#pragma unroll
+      for (int q = 0; q < 4 * MB; ++q)
+        bias4[q] = Tr::lds_read_tr(reinterpret_cast<const T*>(Bt + (32 * (q / 4) + 8 * (q % 4)) * SM::BIAS_STR));
+    }
     const char* Vt = smem_raw + SM::V_OFF;
     op_t vl[3];          // ring of V operands when they come from LDS
     if (kVLds) {
@@ -446,9 +459,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
       float x;
       if (kBias) {
-        // rows of a full tile are all inside the sequence; offsets inside a tile fit 32 bits
-        const int ml = 32 * mb + 8 * g + r;
-        const float bv = (float)Bs[(ml + 4 * hi) * (SM::BIAS_STR / 2)];
+        const float bv = (float)bias4[E / 4][r];
         x = __builtin_fmaf(s[mb][i], qk_scale, bv * kLog2e) - l4[(E / 4) & 1][r];
       } else {
         x = __builtin_fmaf(s[mb][i], qk_scale, -l4[(E / 4) & 1][r]);
