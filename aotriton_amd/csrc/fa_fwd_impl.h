@@ -109,7 +109,14 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   constexpr int LPRQ = D / 8;             // 16-byte pieces per row
   constexpr int RPQ = 64 / LPRQ;          // rows per wave-wide access
   char* rowbuf = smem_raw + SM::ROWS_OFF + wave * 32 * SM::ROW_STR;
-  const int wrows = si.seqlen_q - q0 - wave * 32 < 32 ? si.seqlen_q - q0 - wave * 32 : 32;   // may be <= 0
+  // The descriptors of the wave's Q and O rows are built from a scalar copy of the wave index.
+  // With the per-lane one the compiler takes them for divergent and wraps every access in a loop
+  // over the distinct descriptors (readfirstlane, compare, masked issue): 8-16 such loops per item,
+  // and a register spilled next to one of them was stored while no lane was enabled (the loop
+  // leaves exec at zero and the spill landed before exec is restored), so that the fourth Q piece
+  // of a D = 64 bias + dropout build was fetched from wherever the slot's old content pointed.
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wrows = si.seqlen_q - q0 - wave_u * 32 < 32 ? si.seqlen_q - q0 - wave_u * 32 : 32;   // may be <= 0
   const int rq = lane / LPRQ, cq = lane % LPRQ;
   const T* kbase = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
                    (int64_t)hk * a.sk.h + (int64_t)si.k_start * a.sk.s;
@@ -171,7 +178,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   op_t qreg[KS];
   {
     const T* qw = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
-                  (int64_t)(si.q_start + q0 + wave * 32) * a.sq.s;
+                  (int64_t)(si.q_start + q0 + wave_u * 32) * a.sq.s;
     const auto qrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qw), 0,
                                                        wrows > 0 ? ((wrows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
     const int qvoff = cq * 8 < d_qk ? rq * (int)a.sq.s * 2 + cq * 16 : kVoffOutOfRange;
@@ -250,6 +257,44 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 
   f32x16 s[MB];   // S^T of the current tile
 
+  // Bias tiles of the wave (32 rows x BN keys) travel as row-contiguous 16-byte pieces, consecutive
+  // lanes along a row, and change to the one-row-per-lane layout of S^T in the wave's row area,
+  // which is idle between the Q rows at the start and the O rows at the end of an item.  (One
+  // 8-byte load per lane and 4 keys touches 32 cache lines for 16 bytes each; the vector memory
+  // pipe's line rate then costs more than the bias bytes.)  A row of the area holds D keys, so a
+  // tile passes in BN / BCK chunks of BCK keys.  The pieces are requested behind the QK MFMAs, not
+  // before them: 16 more live registers across that phase cost the causal kernel more in spills
+  // than the exposed latency costs with two waves per SIMD.
+  constexpr int BCK = BN < D ? BN : D;    // keys per chunk
+  constexpr int BLPR = BCK / 8;           // 16-byte pieces per chunk row
+  constexpr int BRPI = 64 / BLPR;         // rows per wave-wide access
+  constexpr int BNI = 32 / BRPI;          // accesses per chunk
+  const int brow = lane / BLPR, bch = lane % BLPR;
+  const bool bias_co = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 7) == 0 &&
+                       (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0;
+  // adds chunk `ck` of tile j's bias to s (the tile lies inside the key range)
+  auto bias_chunk = [&](int j, int ck) {
+    const T* bh = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)h * a.sb_h;
+    op_t bco[BNI];
+#pragma unroll
+    for (int i = 0; i < BNI; ++i) {
+      int m = q0 + wave * 32 + brow + BRPI * i;
+      m = m < si.seqlen_q ? m : si.seqlen_q - 1;
+      bco[i] = *reinterpret_cast<const op_t*>(bh + (int64_t)m * a.sb_m + j * BN + ck * BCK + bch * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < BNI; ++i)
+      *reinterpret_cast<op_t*>(rowbuf + (brow + BRPI * i) * SM::ROW_STR + bch * 16) = bco[i];
+#pragma unroll
+    for (int mbl = 0; mbl < BCK / 32; ++mbl)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const q4_t b4 = *reinterpret_cast<const q4_t*>(rowbuf + c * SM::ROW_STR + (mbl * 32 + 8 * g + 4 * hi) * 2);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[ck * (BCK / 32) + mbl][4 * g + r] += (float)b4[r] * kLog2e;   // fwd_kernel_inner.py:187
+      }
+  };
+
   auto qk = [&](int stage) {
     const T* ks = Ks + stage * SM::K_ELEMS + c * KSTR + hi * 8;
 #pragma unroll
@@ -288,7 +333,10 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
         for (int i = 0; i < 16; ++i) s[mb][i] *= qk_scale;
     }
     if (kBias) {
-      if (bias_vec && (j + 1) * BN <= si.seqlen_k) {
+      if (bias_co && (j + 1) * BN <= si.seqlen_k) {
+#pragma unroll
+        for (int ck = 0; ck < BN / BCK; ++ck) bias_chunk(j, ck);
+      } else if (bias_vec && (j + 1) * BN <= si.seqlen_k) {
         // a lane's four consecutive keys of every 8-key group in one 8-byte load
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -489,7 +537,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     }
   {
     T* ow = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
-            (int64_t)(si.q_start + q0 + wave * 32) * a.so.s;
+            (int64_t)(si.q_start + q0 + wave_u * 32) * a.so.s;
     const auto ors = __builtin_amdgcn_make_buffer_rsrc(ow, 0, wrows > 0 ? ((wrows - 1) * (int)a.so.s + d_v) * 2 : 0,
                                                        0x00020000);
     const int ovoff = cq * 8 < d_v ? rq * (int)a.so.s * 2 + cq * 16 : kVoffOutOfRange;

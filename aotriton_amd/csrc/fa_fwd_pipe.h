@@ -289,7 +289,15 @@ __device__ __forceinline__ void fwd_item_pipe(const FwdArgs& a, const int z, con
   // 8-byte bias loads need unit column stride and 8-byte aligned rows
   const bool bias_vec = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 3) == 0 &&
                         (reinterpret_cast<uintptr_t>(a.bias) & 7) == 0;
-  q4_t bin[QB][4], bout[QB][4];   // bias of the unit before this one / of this one (fetched one step ahead)
+  // Bias of a unit: fetched one step ahead as row-contiguous 16-byte pieces (4 lanes along a row of
+  // 32 keys, 16 rows per wave-wide access: one 8-byte load per lane and 4 keys would touch 32 cache
+  // lines for 16 bytes each), turned into the one-row-per-lane layout in the wave's row area, which
+  // is idle between the Q rows at the start and the O rows at the end of an item.
+  constexpr int BNI = RW / 16;    // accesses per unit
+  q4_t bin[QB][4];                // bias of the unit before this one, in the layout of S^T
+  op_t bco[BNI];                  // pieces of this unit's bias on their way in
+  const bool bias_co = kBias && a.sb_n == 1 && ((a.sb_m | a.sb_h | a.sb_z) & 7) == 0 &&
+                       (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0;
 
   DropoutState ds{};
   if (kDropout) ds = make_dropout(a.drop, z, h, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
@@ -408,11 +416,14 @@ __device__ __forceinline__ void fwd_item_pipe(const FwdArgs& a, const int z, con
 
   // bias of unit g, used by the step after it
   auto fetch_bias = [&](int g) {
-    if (kBias && bias_vec && g <= u1 && (g + 1) * 32 <= si.seqlen_k) {
+    if (kBias && bias_co && g <= u1 && (g + 1) * 32 <= si.seqlen_k) {
+      const T* bh = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)h * a.sb_h;
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) bout[qb][q] = *reinterpret_cast<const q4_t*>(bptr[qb] + g * 32 + 8 * q + 4 * hi);
+      for (int i = 0; i < BNI; ++i) {
+        int m = w_rmin + lane / 4 + 16 * i;
+        m = m < si.seqlen_q ? m : si.seqlen_q - 1;
+        bco[i] = *reinterpret_cast<const op_t*>(bh + (int64_t)m * a.sb_m + g * 32 + (lane % 4) * 8);
+      }
     }
   };
   // what a step leaves to the next one
@@ -422,10 +433,17 @@ __device__ __forceinline__ void fwd_item_pipe(const FwdArgs& a, const int z, con
       x[qb] = acc[qb];
       pin[qb][0] = pout[qb][0];
       pin[qb][1] = pout[qb][1];
-      if (kBias) {
+    }
+    if (kBias && bias_co) {
+      // (pieces that were not fetched carry leftovers; the step that would use them is not speculative)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) bin[qb][q] = bout[qb][q];
-      }
+      for (int i = 0; i < BNI; ++i)
+        *reinterpret_cast<op_t*>(rowbuf + (lane / 4 + 16 * i) * SM::ROW_STR + (lane % 4) * 16) = bco[i];
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          bin[qb][q] = *reinterpret_cast<const q4_t*>(rowbuf + (qb * 32 + c) * SM::ROW_STR + (8 * q + 4 * hi) * 2);
     }
   };
   // a unit past the wave's last one (or no unit at all) contributes P = 0
@@ -528,7 +546,7 @@ __device__ __forceinline__ void fwd_item_pipe(const FwdArgs& a, const int z, con
   };
   // unit g-1 may take the speculative step (given a reference in every row)
   auto spec_ok = [&](int g) -> bool {
-    return g <= u1 && unit_sees_all(g - 1) && (kBias ? bias_vec : !prescale);
+    return g <= u1 && unit_sees_all(g - 1) && (kBias ? bias_co : !prescale);
   };
 
   // ---- main loop ---------------------------------------------------------------------------------------------
