@@ -90,9 +90,50 @@ def build(jobs=8, force=False, verbose=True):
     return LIB
 
 
+_WATERFALL = re.compile(r'v_readfirstlane_b32[^\n]*\n(?:[^\n]*\n){0,24}?[^\n]*s_and_saveexec_b64[^\n]*\n'
+                        r'(?:[^\n]*\n){0,24}?[^\n]*buffer_(?:load|store)[^\n]*\n(?:[^\n]*\n){0,4}?'
+                        r'[^\n]*s_xor_b64 exec, exec[^\n]*\n[^\n]*s_cbranch_execnz')
+
+
+def scan(jobs=8):
+    """Compiles every kernel file to assembly and reports per-descriptor loops around buffer
+    accesses ("waterfall" loops: readfirstlane, compare, masked issue, repeat while lanes are left).
+    The compiler emits them when it takes a buffer descriptor for divergent, e.g. one built from
+    threadIdx.x >> 6.  They cost time, and hipcc 7.2 has placed a register spill in the block such
+    a loop exits to, before exec is restored: the store runs with no lane enabled and the reload
+    later returns whatever the slot held.  The kernels here are written so that none is emitted;
+    returns the list of (file, loops, functions left out of line) that have some of either."""
+    tmp = os.path.join(OBJ, 'scan')
+    os.makedirs(tmp, exist_ok=True)
+
+    def one(unit):
+        src, defines, objname = unit
+        if not src.endswith('.hip'):
+            return src, 0, 0
+        out = os.path.join(tmp, objname + '.s')
+        cmd = [HIPCC] + COMMON + EXTRA.get(src, []) + defines + ['-x', 'hip', '--cuda-device-only', '-S',
+                                                                 os.path.join(CSRC, src), '-o', out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError('hipcc failed on ' + src)
+        text = open(out).read()
+        # a device function left out of line (a lambda the inliner gave up on) keeps its captures in
+        # memory and reads them back with flat loads; every kernel here is meant to be one function
+        outlined = len(re.findall(r'^\s*\.type\s+\S+,@function', text, re.M)) - text.count('.amdhsa_kernel ')
+        return objname, len(_WATERFALL.findall(text)), outlined
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        return [(n, c, o) for n, c, o in ex.map(one, sources()) if c or o]
+
+
 if __name__ == '__main__':
     ap = argparse.ArgumentParser()
     ap.add_argument('-j', type=int, default=8)
     ap.add_argument('--force', action='store_true')
+    ap.add_argument('--scan', action='store_true', help='compile to assembly and look for per-descriptor loops')
     a = ap.parse_args()
+    if a.scan:
+        found = scan(a.j)
+        print('per-descriptor loops / functions left out of line:', found if found else 'none')
+        sys.exit(1 if found else 0)
     print(build(a.j, a.force))

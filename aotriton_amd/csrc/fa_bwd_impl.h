@@ -191,9 +191,30 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   // the last tile into a no-op.
   static_assert(NCH % NT == 0, "threads must cover the tile evenly");
   constexpr int RPI = NT / LPR;                  // rows between two pieces of one thread
-  op_t qch[CH], doch[CH], och[kInlineDelta ? CH : 1];
+  // D = 256: the Q and dO pieces go from global memory straight into the LDS stage (no staging
+  // registers: next to 256 accumulators, the K operands and the softmax state they were what
+  // pushed the K operands out to scratch, and a scratch reload waits for every load in flight).
+  // A wave instruction fills 1 KB of consecutive LDS, two rows; the swizzle is applied on the
+  // global side: the lane at chunk position p of row r fetches chunk p ^ f(r).
+  constexpr bool kDirect = D >= 256 && !kInlineDelta;
+  op_t qch[kDirect ? 1 : CH], doch[kDirect ? 1 : CH], och[kInlineDelta ? CH : 1];
   float l_stage = 0.f, d_stage = 0.f;
   const int r0 = tid / LPR, cc0 = tid % LPR;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int f_stage = 0;                               // stage the running fetch fills
+  // f(r0 + k RPI) takes two values, for even and odd k (RPI = 8: the row's bits 0-2 are r0's)
+  int q_voff_d[2] = {0, 0}, do_voff_d[2] = {0, 0};
+  if (kDirect) {
+    static_assert(!kDirect || (LPR == 32 && RPI == 8 && CH % 2 == 0), "direct staging assumes 512-byte rows");
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int gch = cc0 ^ Swz<D>::f(r0 + k * RPI);
+      q_voff_d[k] = gch * 8 < d_qk ? r0 * (int)a.sq.s * 2 + gch * 16 : kVoffOutOfRange;
+      do_voff_d[k] = gch * 8 < d_v ? r0 * (int)a.sdo.s * 2 + gch * 16 : kVoffOutOfRange;
+    }
+  }
+  BufDesc q_dd{}, do_dd{};
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem_raw;
   const int q_voff = cc0 * 8 < d_qk ? r0 * (int)a.sq.s * 2 + cc0 * 16 : kVoffOutOfRange,       // bytes inside a tile
             do_voff = cc0 * 8 < d_v ? r0 * (int)a.sdo.s * 2 + cc0 * 16 : kVoffOutOfRange,
             o_voff = cc0 * 8 < d_v ? r0 * (int)a.so.s * 2 + cc0 * 16 : kVoffOutOfRange;
@@ -254,10 +275,15 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
                                                any && bias_lds ? ((rows - 1) * (int)a.sb_m + b_cols) * 2 : 0, 0x00020000);
       if (live) bb += (int64_t)BM * a.sb_m;
     }
-    q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0,
-                                             0x00020000);
-    do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
-                                              any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0, 0x00020000);
+    if constexpr (kDirect) {
+      q_dd = make_buf_desc(qb, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0);
+      do_dd = make_buf_desc(dob, any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0);
+    } else {
+      q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0,
+                                               any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
+      do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
+                                                any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0, 0x00020000);
+    }
     if (kInlineDelta)
       o_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ob), 0,
                                                any ? ((rows - 1) * (int)a.so.s + d_v) * 2 : 0, 0x00020000);
@@ -304,13 +330,28 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         bch[k] = x;
       }
     } else if (i < CH) {
-      qch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(q_rs, q_voff, i * q_soff, 0));
+      if constexpr (kDirect) {
+        buffer_load_lds16(q_dd, lds0 + f_stage * SM::STAGE_BYTES + (i * RPI + 2 * wave_u) * Swz<D>::ROWB,
+                          q_voff_d[i & 1], i * q_soff);
+      } else {
+        qch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(q_rs, q_voff, i * q_soff, 0));
+      }
     } else {
       const int k = i - CH;
-      doch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(do_rs, do_voff, k * do_soff, 0));
+      if constexpr (kDirect) {
+        buffer_load_lds16(do_dd,
+                          lds0 + f_stage * SM::STAGE_BYTES + SM::TILE_BYTES + (k * RPI + 2 * wave_u) * Swz<D>::ROWB,
+                          do_voff_d[k & 1], k * do_soff);
+      } else {
+        doch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(do_rs, do_voff, k * do_soff, 0));
+      }
       if (kInlineDelta)
         och[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(o_rs, o_voff, k * o_soff, 0));
     }
+  };
+  // all of this wave's direct pieces have landed (vmcnt 0; the other counters stay as they are)
+  auto direct_landed = [&]() {
+    if constexpr (kDirect) __builtin_amdgcn_s_waitcnt(0x0F70);
   };
   constexpr int STORE_PIECES = 2 * CH + CHB;
   auto store_piece = [&](int i, int stage) {   // same order as the fetches
@@ -318,6 +359,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     if (i >= 2 * CH)
       *reinterpret_cast<op_t*>(sp + 2 * SM::TILE_BYTES + 2 * BM * 4 + b_lds + (i - 2 * CH) * (NT / 16) * SM::BIAS_STR) =
           bch[i - 2 * CH];
+    else if (kDirect) return;
     else if (i < CH) *reinterpret_cast<op_t*>(sp + lds_off[i]) = qch[i];
     else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = doch[i - CH];
   };
@@ -409,7 +451,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         // the next tile's descriptors and global loads ride behind these MFMAs
         constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
         const int gidx = k * MB + mb;
-        if (gidx == 0) fetch_begin(live, g_nxt, e_nxt);
+        if (gidx == 0) { f_stage = stage ^ 1; fetch_begin(live, g_nxt, e_nxt); }
         if (kDropout) {
           // One Philox call yields the keep bits of 4 consecutive keys, i.e. of the 4
           // lanes of a quad, for one row: quad lane q runs the calls of the rows with
@@ -434,11 +476,19 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     }
     // row statistics of the tile's queries and the first dO operands
     l4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ls, 0));
-    typename Tr::q4_t bias4[kBias ? 4 * MB : 1];
+    // D = 256 has no registers for the whole column: there the reads run one ahead of their use
+    constexpr bool kBiasRing = D >= 256;
+    typename Tr::q4_t bias4[kBias ? (kBiasRing ? 2 : 4 * MB) : 1];
+    auto bias_read = [&](int q) {
+      return Tr::lds_read_tr(reinterpret_cast<const T*>(Bt + (32 * (q / 4) + 8 * (q % 4)) * SM::BIAS_STR));
+    };
     if (kBias) {
+      if (kBiasRing) {
+        bias4[0] = bias_read(0);
+      } else {
 #pragma unroll
-      for (int q = 0; q < 4 * MB; ++q)
-        bias4[q] = Tr::lds_read_tr(reinterpret_cast<const T*>(Bt + (32 * (q / 4) + 8 * (q % 4)) * SM::BIAS_STR));
+        for (int q = 0; q < 4 * MB; ++q) bias4[q] = bias_read(q);
+      }
     }
     const char* Vt = smem_raw + SM::V_OFF;
     op_t vl[3];          // ring of V operands when they come from LDS
@@ -459,7 +509,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
       float x;
       if (kBias) {
-        const float bv = (float)bias4[E / 4][r];
+        if (kBiasRing && E % 4 == 0 && E + 4 < 16 * MB) bias4[(E / 4 + 1) & 1] = bias_read(E / 4 + 1);
+        const float bv = (float)bias4[kBiasRing ? (E / 4) & 1 : E / 4][r];
         x = __builtin_fmaf(s[mb][i], qk_scale, bv * kLog2e) - l4[(E / 4) & 1][r];
       } else {
         x = __builtin_fmaf(s[mb][i], qk_scale, -l4[(E / 4) & 1][r]);
@@ -632,6 +683,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       __builtin_amdgcn_sched_barrier(0);
     }
     store_stats(stage ^ 1);
+    direct_landed();
   };
 
   if (kVLds) {
@@ -656,6 +708,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 #pragma unroll
   for (int i = 0; i < STORE_PIECES; ++i) store_piece(i, 0);
   store_stats(0);
+  direct_landed();
   __syncthreads();
   // Per q-head the Q tiles come as [masked | full | masked]; each run has its own
   // loop so that the loop bodies are straight-line code.
@@ -927,7 +980,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   // element code then has no run-time branch.  Other tiles of a bias run take the general code, in a
   // loop of their own: one loop body holding both would branch around every element and move the
   // accumulators between the two copies of its MFMAs.
-  auto compute = [&](auto masked_tag, auto fast_tag, int j, int stage, bool live) {
+  auto compute = [&](auto masked_tag, auto fast_tag, int j, int stage, bool live) __attribute__((always_inline)) {
     constexpr bool masked = decltype(masked_tag)::value;
     constexpr bool kFast = decltype(fast_tag)::value;
     constexpr int G1 = KS * MB, G4 = TS * DB;
@@ -1124,7 +1177,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   // K tiles come as [masked | full | masked]; one straight-line loop per run
   {
     int j = br.lo;
-    auto step = [&](auto masked_tag, auto fast_tag) {
+    auto step = [&](auto masked_tag, auto fast_tag) __attribute__((always_inline)) {
       const int stage = (j - br.lo) & 1;
       compute(masked_tag, fast_tag, j, stage, j < br.hi);
       __syncthreads();
@@ -1134,7 +1187,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     const int full_hi = br.fb_lo <= br.fb_hi ? br.fb_hi : br.hi;
     // last tile that lies inside the key range (the vector code of a bias run ends there)
     const int j_in = item_fast ? si.seqlen_k / BN - 1 : br.lo - 1;
-    auto run = [&](auto masked_tag, int upto) {
+    // (a closure left out of line keeps its captures in memory: every use becomes a flat load)
+    auto run = [&](auto masked_tag, int upto) __attribute__((always_inline)) {
       if constexpr (kBias) {
         const int fast_to = upto < j_in ? upto : j_in;
         while (j <= fast_to) step(masked_tag, std::true_type{});
