@@ -195,7 +195,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   // registers: next to 256 accumulators, the K operands and the softmax state they were what
   // pushed the K operands out to scratch, and a scratch reload waits for every load in flight).
   // A wave instruction fills 1 KB of consecutive LDS, two rows; the swizzle is applied on the
-  // global side: the lane at chunk position p of row r fetches chunk p ^ f(r).
+  // global side: the lane at chunk position p of row r fetches chunk p ^ f(r).  Lanes outside the
+  // descriptor's range deliver zeros.  The pieces count in vmcnt like any load; the compiler makes
+  // the first transposing LDS read after them wait for all of them (mid-tile: they have landed).
   constexpr bool kDirect = D >= 256 && !kInlineDelta;
   op_t qch[kDirect ? 1 : CH], doch[kDirect ? 1 : CH], och[kInlineDelta ? CH : 1];
   float l_stage = 0.f, d_stage = 0.f;
@@ -213,8 +215,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       do_voff_d[k] = gch * 8 < d_v ? r0 * (int)a.sdo.s * 2 + gch * 16 : kVoffOutOfRange;
     }
   }
-  BufDesc q_dd{}, do_dd{};
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem_raw;
+  using lds_ptr_t = __attribute__((address_space(3))) void*;
   const int q_voff = cc0 * 8 < d_qk ? r0 * (int)a.sq.s * 2 + cc0 * 16 : kVoffOutOfRange,       // bytes inside a tile
             do_voff = cc0 * 8 < d_v ? r0 * (int)a.sdo.s * 2 + cc0 * 16 : kVoffOutOfRange,
             o_voff = cc0 * 8 < d_v ? r0 * (int)a.so.s * 2 + cc0 * 16 : kVoffOutOfRange;
@@ -275,15 +276,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
                                                any && bias_lds ? ((rows - 1) * (int)a.sb_m + b_cols) * 2 : 0, 0x00020000);
       if (live) bb += (int64_t)BM * a.sb_m;
     }
-    if constexpr (kDirect) {
-      q_dd = make_buf_desc(qb, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0);
-      do_dd = make_buf_desc(dob, any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0);
-    } else {
-      q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0,
-                                               any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
-      do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
-                                                any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0, 0x00020000);
-    }
+    q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0,
+                                             0x00020000);
+    do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
+                                              any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0, 0x00020000);
     if (kInlineDelta)
       o_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ob), 0,
                                                any ? ((rows - 1) * (int)a.so.s + d_v) * 2 : 0, 0x00020000);
@@ -331,17 +327,18 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       }
     } else if (i < CH) {
       if constexpr (kDirect) {
-        buffer_load_lds16(q_dd, lds0 + f_stage * SM::STAGE_BYTES + (i * RPI + 2 * wave_u) * Swz<D>::ROWB,
-                          q_voff_d[i & 1], i * q_soff);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            q_rs, (lds_ptr_t)(stage_ptr(f_stage) + (i * RPI + 2 * wave_u) * Swz<D>::ROWB), 16, q_voff_d[i & 1],
+            i * q_soff, 0, 0);
       } else {
         qch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(q_rs, q_voff, i * q_soff, 0));
       }
     } else {
       const int k = i - CH;
       if constexpr (kDirect) {
-        buffer_load_lds16(do_dd,
-                          lds0 + f_stage * SM::STAGE_BYTES + SM::TILE_BYTES + (k * RPI + 2 * wave_u) * Swz<D>::ROWB,
-                          do_voff_d[k & 1], k * do_soff);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            do_rs, (lds_ptr_t)(stage_ptr(f_stage) + SM::TILE_BYTES + (k * RPI + 2 * wave_u) * Swz<D>::ROWB), 16,
+            do_voff_d[k & 1], k * do_soff, 0, 0);
       } else {
         doch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(do_rs, do_voff, k * do_soff, 0));
       }

@@ -275,28 +275,6 @@ __device__ __forceinline__ SeqInfo get_seq(const SeqArgs& s, int z) {
 // chunk lies in the padding of a head dim that was rounded up reads zeros with it.
 constexpr int kVoffOutOfRange = 0x7fff0000;
 
-// Buffer load of 16 bytes per lane straight into LDS: lane L's piece lands at lds_base + 16 L (a
-// wave instruction fills 1 KB of consecutive LDS), lanes outside the descriptor's range deliver
-// zeros.  Counted by vmcnt like any load; the compiler is not told that LDS is written (it would
-// wait for every piece in flight before the next transposing LDS read), so the caller waits for
-// vmcnt(0) before the barrier that publishes the tile.
-struct BufDesc { vec<int, 4> w; };
-__device__ __forceinline__ BufDesc make_buf_desc(const void* base, int bytes) {
-  const uint64_t p = reinterpret_cast<uint64_t>(base);
-  BufDesc d;
-  d.w[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
-  d.w[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32) & 0xffff);
-  d.w[2] = __builtin_amdgcn_readfirstlane(bytes);
-  d.w[3] = 0x00020000;
-  return d;
-}
-__device__ __forceinline__ void buffer_load_lds16(const BufDesc& d, uint32_t lds_base, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(d.w), "s"(soff)
-               : "memory", "m0");
-}
-
 // (sequence, head) of the linear work index zh.  The heads of one GQA group are
 // adjacent, then come the sequences, then the kv-heads: the contiguous range of zh
 // that an XCD owns then holds whole kv-heads across ALL sequences, so XCDs get equal
