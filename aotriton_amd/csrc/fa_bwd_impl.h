@@ -191,23 +191,26 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   // the last tile into a no-op.
   static_assert(NCH % NT == 0, "threads must cover the tile evenly");
   constexpr int RPI = NT / LPR;                  // rows between two pieces of one thread
-  // D = 256: the Q and dO pieces go from global memory straight into the LDS stage (no staging
-  // registers: next to 256 accumulators, the K operands and the softmax state they were what
-  // pushed the K operands out to scratch, and a scratch reload waits for every load in flight).
-  // A wave instruction fills 1 KB of consecutive LDS, two rows; the swizzle is applied on the
+  // The Q and dO pieces go from global memory straight into the LDS stage (no staging registers
+  // and no LDS write instructions: 3-5 % at D = 64 and 128; at D = 256 the staging registers,
+  // next to 256 accumulators, the K operands and the softmax state, were what pushed the K
+  // operands out to scratch, and a scratch reload waits for every load in flight).  A wave
+  // instruction fills 1 KB of consecutive LDS, 64 / LPR rows; the swizzle is applied on the
   // global side: the lane at chunk position p of row r fetches chunk p ^ f(r).  Lanes outside the
   // descriptor's range deliver zeros.  The pieces count in vmcnt like any load; the compiler makes
   // the first transposing LDS read after them wait for all of them (mid-tile: they have landed).
-  constexpr bool kDirect = D >= 256 && !kInlineDelta;
+  // The fused kernel computes delta from the staged O and dO registers and keeps them.
+  constexpr bool kDirect = !kInlineDelta;
+  constexpr int RWI = 64 / LPR;                  // rows one wave instruction covers
   op_t qch[kDirect ? 1 : CH], doch[kDirect ? 1 : CH], och[kInlineDelta ? CH : 1];
   float l_stage = 0.f, d_stage = 0.f;
   const int r0 = tid / LPR, cc0 = tid % LPR;
   const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
   int f_stage = 0;                               // stage the running fetch fills
-  // f(r0 + k RPI) takes two values, for even and odd k (RPI = 8: the row's bits 0-2 are r0's)
+  // f(r0 + k RPI) takes at most two values, for even and odd k (RPI is a multiple of 8, f has period 16)
   int q_voff_d[2] = {0, 0}, do_voff_d[2] = {0, 0};
   if (kDirect) {
-    static_assert(!kDirect || (LPR == 32 && RPI == 8 && CH % 2 == 0), "direct staging assumes 512-byte rows");
+    static_assert(!kDirect || RPI % 8 == 0, "the swizzle must repeat every two pieces");
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const int gch = cc0 ^ Swz<D>::f(r0 + k * RPI);
@@ -328,7 +331,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     } else if (i < CH) {
       if constexpr (kDirect) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            q_rs, (lds_ptr_t)(stage_ptr(f_stage) + (i * RPI + 2 * wave_u) * Swz<D>::ROWB), 16, q_voff_d[i & 1],
+            q_rs, (lds_ptr_t)(stage_ptr(f_stage) + (i * RPI + RWI * wave_u) * Swz<D>::ROWB), 16, q_voff_d[i & 1],
             i * q_soff, 0, 0);
       } else {
         qch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(q_rs, q_voff, i * q_soff, 0));
@@ -337,7 +340,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       const int k = i - CH;
       if constexpr (kDirect) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            do_rs, (lds_ptr_t)(stage_ptr(f_stage) + SM::TILE_BYTES + (k * RPI + 2 * wave_u) * Swz<D>::ROWB), 16,
+            do_rs, (lds_ptr_t)(stage_ptr(f_stage) + SM::TILE_BYTES + (k * RPI + RWI * wave_u) * Swz<D>::ROWB), 16,
             do_voff_d[k & 1], k * do_soff, 0, 0);
       } else {
         doch[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(do_rs, do_voff, k * do_soff, 0));
@@ -931,8 +934,25 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   constexpr int LPR = D / 8;                     // 16-byte pieces per row
   constexpr int RPI = NT / LPR;                  // rows between two pieces of one thread
   static_assert((BN * D / 8) % NT == 0 && NT % LPR == 0, "threads must cover the tile evenly");
-  op_t kch[CH], vch[CH];
+  // (the pieces go straight into the LDS stage, as in the dK/dV item: lane at chunk position p of
+  // row r fetches chunk p ^ f(r), a wave instruction fills 64 / LPR consecutive rows)
+  constexpr bool kDirect = true;
+  constexpr int RWI = 64 / LPR;
+  static_assert(!kDirect || RPI % 8 == 0, "the swizzle must repeat every two pieces");
+  op_t kch[kDirect ? 1 : CH], vch[kDirect ? 1 : CH];
   const int r0 = tid / LPR, cc0 = tid % LPR;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int f_stage = 0;                               // stage the running fetch fills
+  int k_voff_d[2] = {0, 0}, v_voff_d[2] = {0, 0};
+  if (kDirect) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int gch = cc0 ^ Swz<D>::f(r0 + k * RPI);
+      k_voff_d[k] = gch * 8 < d_qk ? r0 * (int)a.sk.s * 2 + gch * 16 : kVoffOutOfRange;
+      v_voff_d[k] = gch * 8 < d_v ? r0 * (int)a.sv.s * 2 + gch * 16 : kVoffOutOfRange;
+    }
+  }
+  using lds_ptr_t = __attribute__((address_space(3))) void*;
   const int k_voff = cc0 * 8 < d_qk ? r0 * (int)a.sk.s * 2 + cc0 * 16 : kVoffOutOfRange,
             v_voff = cc0 * 8 < d_v ? r0 * (int)a.sv.s * 2 + cc0 * 16 : kVoffOutOfRange;
   const int k_soff = RPI * (int)a.sk.s * 2, v_soff = RPI * (int)a.sv.s * 2;
@@ -960,15 +980,31 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   };
   constexpr int FETCH_PIECES = 2 * CH;
   auto fetch_piece = [&](int i) {        // K pieces first, then V
-    if (i < CH)
-      kch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff, i * k_soff, 0));
-    else
-      vch[i - CH] =
-          __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_voff, (i - CH) * v_soff, 0));
+    if constexpr (kDirect) {
+      char* sp = smem_raw + f_stage * SM::STAGE_BYTES;
+      if (i < CH)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rs, (lds_ptr_t)(sp + (i * RPI + RWI * wave_u) * Swz<D>::ROWB), 16,
+                                                 k_voff_d[i & 1], i * k_soff, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            v_rs, (lds_ptr_t)(sp + SM::TILE_BYTES + ((i - CH) * RPI + RWI * wave_u) * Swz<D>::ROWB), 16,
+            v_voff_d[(i - CH) & 1], (i - CH) * v_soff, 0, 0);
+    } else {
+      if (i < CH)
+        kch[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff, i * k_soff, 0));
+      else
+        vch[i - CH] =
+            __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_voff, (i - CH) * v_soff, 0));
+    }
+  };
+  // all of this wave's direct pieces have landed (vmcnt 0; the other counters stay as they are)
+  auto direct_landed = [&]() {
+    if constexpr (kDirect) __builtin_amdgcn_s_waitcnt(0x0F70);
   };
   constexpr int STORE_PIECES = 2 * CH;
   auto store_piece = [&](int i, int stage) {   // same order as the fetches
     char* sp = smem_raw + stage * SM::STAGE_BYTES;
+    if (kDirect) return;
     if (i < CH) *reinterpret_cast<op_t*>(sp + lds_off[i]) = kch[i];
     else *reinterpret_cast<op_t*>(sp + SM::TILE_BYTES + lds_off[i - CH]) = vch[i - CH];
   };
@@ -1031,7 +1067,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         constexpr int every = G1 / FETCH_PIECES > 0 ? G1 / FETCH_PIECES : 1;
         constexpr int per = (FETCH_PIECES + G1 - 1) / G1;
         const int gidx = k * MB + mb;
-        if (gidx == 0) fetch_begin(live);
+        if (gidx == 0) { f_stage = stage ^ 1; fetch_begin(live); }
         if (gidx % every == every - 1) {
 #pragma unroll
           for (int q = 0; q < per; ++q) {
@@ -1163,6 +1199,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         if (m < si.seqlen_q) *reinterpret_cast<op_t*>(db_head + (int64_t)m * a.sdb_m + j * BN + bch * 8) = x;
       }
     }
+    direct_landed();
   };
 
   fetch_begin(true);
@@ -1170,6 +1207,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   for (int i = 0; i < FETCH_PIECES; ++i) fetch_piece(i);
 #pragma unroll
   for (int i = 0; i < STORE_PIECES; ++i) store_piece(i, 0);
+  direct_landed();
   __syncthreads();
   // K tiles come as [masked | full | masked]; one straight-line loop per run
   {
