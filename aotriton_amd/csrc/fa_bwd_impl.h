@@ -152,6 +152,17 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     return;
   }
 
+  // Queries that see this lane's key form one range [q_lo, q_lo + q_rng] (none: q_none): a masked
+  // tile then tests an element with one unsigned comparison (fwd_kernel_inner.py:140-160 states the
+  // predicate per element: key <= m + right, key >= m - left, both inside their sequences).
+  int q_lo = 0, q_hi = si.seqlen_q - 1;
+  if (kWindowed) {
+    q_lo = key - w.right > 0 ? key - w.right : 0;
+    q_hi = key + w.left < q_hi ? key + w.left : q_hi;
+  }
+  const bool q_none = !key_ok || q_hi < q_lo;
+  const unsigned q_rng = q_none ? 0u : (unsigned)(q_hi - q_lo);
+
   // K and V rows of this lane's key as B operands (k = head dim)
   const T* kptr = reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z + (int64_t)hk * a.sk.h +
                   (int64_t)(si.k_start + key_c) * a.sk.s;
@@ -502,9 +513,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(dOb, row_a, k, mb);
 
     // element E = 16*mb + i of the tile: p (kept in s, undropped) and its operand form
+    const unsigned q_d = q_none ? 0x40000000u : (unsigned)(m0 + 4 * hi - q_lo);
     auto p_el = [&](int E) {
       const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
-      const int m = m0 + 32 * mb + 8 * g + 4 * hi + r;
       if (E % 4 == 0 && E + 4 < 16 * MB) l4[(E / 4 + 1) & 1] = *reinterpret_cast<const f32x4*>(stat_ptr(Ls, E / 4 + 1));
       // p = exp2(s*c + bias*log2e - L*log2e), one fma per element (bwd_inner_dk_dv.py:187-188)
       float x;
@@ -516,8 +527,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         x = __builtin_fmaf(s[mb][i], qk_scale, -l4[(E / 4) & 1][r]);
       }
       if (masked) {
-        bool vis = (m < si.seqlen_q) & key_ok;
-        if (kWindowed) vis = vis & (key <= m + w.right) & (key >= m - w.left);
+        // query m sees this lane's key iff q_lo <= m <= q_lo + q_rng; an empty range fails every element
+        const bool vis = q_d + (unsigned)(32 * mb + 8 * g + r) <= q_rng;
         x = vis ? x : -__builtin_inff();
       }
       s[mb][i] = fast_exp2(x);
@@ -784,6 +795,15 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   const int row = q0 + wave * 32 + c;
   const bool row_ok = row < si.seqlen_q;
   const int row_c = row_ok ? row : si.seqlen_q - 1;
+
+  // keys visible to this lane's query form one range [m_lo, m_lo + m_rng] (none: m_none)
+  int m_lo = 0, m_hi = si.seqlen_k - 1;
+  if (kWindowed) {
+    m_lo = row - w.left > 0 ? row - w.left : 0;
+    m_hi = row + w.right < m_hi ? row + w.right : m_hi;
+  }
+  const bool m_none = m_hi < m_lo;
+  const unsigned m_rng = m_none ? 0u : (unsigned)(m_hi - m_lo);
 
   T* dqptr = reinterpret_cast<T*>(a.dq) + (int64_t)si.batch_index * a.sdq.z + (int64_t)h * a.sdq.h +
              (int64_t)(si.q_start + row_c) * a.sdq.s;
@@ -1093,6 +1113,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     }
 
     // element E = 16*mb + i of the tile: p, kept in s
+    const unsigned m_d = m_none ? 0x40000000u : (unsigned)(j * BN + 4 * hi - m_lo);
     auto p_el = [&](int E) {
       const int mb = E / 16, i = E % 16, g = i / 4, r = i % 4;
       const int n = j * BN + 32 * mb + 8 * g + 4 * hi + r;
@@ -1110,8 +1131,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         x = __builtin_fmaf(s[mb][i], qk_scale, -l_row);
       }
       if (masked) {
-        bool vis = n < si.seqlen_k;
-        if (kWindowed) vis = vis & (n <= row + w.right) & (n >= row - w.left);
+        // one unsigned comparison of n - m_lo against the length of the visible range
+        const bool vis = m_d + (unsigned)(32 * mb + 8 * g + r) <= m_rng;
         x = vis ? x : -__builtin_inff();
       }
       s[mb][i] = fast_exp2(x);
