@@ -316,7 +316,8 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
-  if (dtype == FA_DTYPE_FLOAT32 || d > 256) return fa::run_fwd_valu(dtype, d, a, stream);
+  if (dtype == FA_DTYPE_FLOAT32) return fa::run_fwd_valu(dtype, d, a, stream);
+  if (d > 256) return fa::run_fwd_d512(dtype, a, s.windowed, s.bias, s.dropout, stream);
   const bool padded = a.head_dim != d || a.head_dim_v != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
     case 64: return (padded ? fa::run_fwd_d64_padded : fa::run_fwd_d64)(dtype, a, s.windowed, s.bias, s.dropout, stream);
@@ -406,8 +407,11 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   Shape s{};
   int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
   if (e != FA_SUCCESS) return e;
-  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
-  const fa::TileShape t = valu ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(params->Q.dtype, s.d, s.windowed);
+  // the vector-ALU kernels (fp32) and the split-head-dim kernels (above 256): 32 rows per workgroup, 3-D grid
+  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;
+  const fa::TileShape t = params->Q.dtype == FA_DTYPE_FLOAT32 ? fa::TileShape{32, 1, 4, 0}
+                          : s.d > 256 ? fa::d512_tile_shape(-1)
+                                      : fa::fwd_tile_shape(params->Q.dtype, s.d, s.windowed);
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
   if (valu) {
@@ -443,8 +447,10 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   if (e != FA_SUCCESS) return e;
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
   if (valu && kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
-  const fa::TileShape t = valu ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
-                               : fa::bwd_tile_shape(params->Q.dtype, s.d, s.windowed, kernel_slot);
+  const bool split_d = params->Q.dtype != FA_DTYPE_FLOAT32 && s.d > 256 && kernel_slot != 0;
+  const fa::TileShape t = split_d ? fa::d512_tile_shape(kernel_slot)
+                          : valu  ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
+                                  : fa::bwd_tile_shape(params->Q.dtype, s.d, s.windowed, kernel_slot);
   const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
@@ -637,13 +643,18 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       }
     }
     a.delta = static_cast<float*>(delta.ptr);
-    const bool f32 = dt == FA_DTYPE_FLOAT32 || s.d > 256;      // vector-ALU kernels
+    const bool f32 = dt == FA_DTYPE_FLOAT32;      // vector-ALU kernels
+    const bool big = !f32 && s.d > 256;           // head dim split over the waves; delta from the vector-ALU kernel
     if (kernel_slot < 0 || kernel_slot == 0)
-      err = f32 ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
+      err = f32 || big ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
     if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 1))
-      err = f32 ? fa::run_bwd_valu(dt, s.d, 1, a, stream) : fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      err = f32   ? fa::run_bwd_valu(dt, s.d, 1, a, stream)
+            : big ? fa::run_bwd_d512(dt, 1, a, s.windowed, s.bias, s.dropout, stream)
+                  : fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 2))
-      err = f32 ? fa::run_bwd_valu(dt, s.d, 2, a, stream) : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      err = f32   ? fa::run_bwd_valu(dt, s.d, 2, a, stream)
+            : big ? fa::run_bwd_d512(dt, 2, a, s.windowed, s.bias, s.dropout, stream)
+                  : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
     if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);   // attn_bwd.cc:157
   } else {
     a.delta = nullptr;

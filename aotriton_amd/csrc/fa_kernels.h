@@ -31,6 +31,13 @@ hipError_t run_bwd_dq(int dtype, int head_dim, const BwdArgs& a, bool windowed, 
 hipError_t run_bwd_fused(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 TileShape bwd_tile_shape(int dtype, int head_dim, bool windowed, int kernel_slot);
 
+// MFMA kernels of the 16-bit types for head dims above 256, rounded up to 512 (the head dim split
+// over the waves of a workgroup).  kernel_slot of the backward: 1 dK/dV, 2 dQ and dB.
+hipError_t run_fwd_d512(int dtype, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_bwd_d512(int dtype, int kernel_slot, const BwdArgs& a, bool windowed, bool bias, bool dropout,
+                        hipStream_t s);
+TileShape d512_tile_shape(int kernel_slot);
+
 // Vector-ALU kernels (no MFMA): fp32 tensors at any head dim, every type at head dim 512.
 // head_dim is the compiled one (64, 128, 256, 512).  kernel_slot of the backward: 0 delta,
 // 1 dK/dV, 2 dQ and dB.
