@@ -156,9 +156,22 @@ def test_fp32_inputs(case):
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize('D,Dv', [(512, None), (320, 264), (128, 512)])
 def test_head_dims_up_to_512(dtype, D, Dv):
-    # above 256 every type runs on the vector-ALU kernels (the reference compiles head dim 512,
-    # modules/flash/aot/_common.py:10-14)
+    # above 256 the 16-bit types run on the kernels that split the head dim over the waves, fp32 on
+    # the vector-ALU kernels (the reference compiles head dim 512, modules/flash/aot/_common.py:10-14)
     _run_case(1, 4, 2, 150, 131, D, dtype, (40, 0), Dv=Dv, bwd_backend=0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('causal', [False, True, (70, 33)])
+@pytest.mark.parametrize('D,Dv,p,bias', [(512, None, 0.0, False), (384, 272, 0.1, False), (264, 512, 0.0, True),
+                                         (448, None, 0.3, True)])
+def test_split_head_dim_kernels(dtype, causal, D, Dv, p, bias):
+    # several tiles of 32 rows each way, ragged ends, grouped heads, every combination of mask,
+    # bias (with dB) and dropout
+    if bias and causal is True:
+        causal = (1000, 0)       # the same mask through the window arguments
+    _run_case(2, 6, 2, 203, 261, D, dtype, causal, Dv=Dv, dropout_p=p, bias=bias, bwd_backend=0)
 
 
 def test_head_dim_512_with_bias_and_dropout():
@@ -212,7 +225,7 @@ def _sampled_grid_cases(n=72, seed=2024):
         p = rnd.choice([0.0, 0.5])
         if p > 0.0 and sq * sk > 600 * 600:
             p = 0.0
-        if max(D, Dv or 0) > 256 and sq * sk > 1024 * 1024:
+        if dtype == torch.float32 and max(D, Dv or 0) > 256 and sq * sk > 1024 * 1024:
             sq, sk = min(sq, 512), min(sk, 512)      # vector-ALU kernels: keep the case short
         split_only = dtype == torch.float32 or max(D, Dv or 0) > 256
         backend = 0 if split_only else rnd.choice([0, 1])
