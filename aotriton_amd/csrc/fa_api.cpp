@@ -415,7 +415,7 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
   if (valu) {
-    out->grid[0] = (s.max_sq + 31) / 32;
+    out->grid[0] = (s.max_sq + t.block_m - 1) / t.block_m;
     out->grid[1] = s.hq;
     out->grid[2] = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
   } else {

@@ -34,14 +34,12 @@ constexpr int kBR = 32;          // rows (queries or keys) per workgroup
 constexpr int kBC = 32;          // rows of the streamed tiles per step
 constexpr int kNT = kNW * 64;
 
-// two streamed tiles per stage: one read by rows (+16 B per row), one read transposed (+64 B per row)
+// padded tiles of the forward: one read by rows (+16 B per row), one read transposed (+64 B per row)
 struct Smem512 {
   static constexpr int ASTR = kD + 8;
   static constexpr int BSTR = kD + 32;
   static constexpr int A_ELEMS = kBC * ASTR;
   static constexpr int B_ELEMS = kBC * BSTR;
-  static constexpr int STAGES = 2;
-  static constexpr int PART_OFF = STAGES * (A_ELEMS + B_ELEMS) * 2;
   static constexpr int PART_BYTES = kNW * 64 * 16 * 4;       // one partial block per wave
 };
 
@@ -71,14 +69,15 @@ __device__ __forceinline__ f32x16 part_sum(const float* area, int lane) {
   return x;
 }
 
-// A tile of kBC rows x 512 columns, global -> registers -> LDS by the whole workgroup: a wave
-// instruction covers one row (64 pieces of 16 bytes), a thread holds 8 pieces 4 rows apart.  The
-// buffer descriptor bounds the tile to its valid rows and columns; what lies outside reads as zero.
-template <typename T>
+// A tile of kBC rows x 512 columns, global -> registers -> LDS by the whole workgroup of NT threads:
+// a wave instruction covers one row (64 pieces of 16 bytes), a thread holds its pieces NT / 64
+// rows apart.  The buffer descriptor bounds the tile to its valid rows and columns; what lies
+// outside reads as zero.
+template <typename T, int NT = kNT>
 struct TileFetch {
   using op_t = typename Traits<T>::op_t;
-  static constexpr int CH = kBC * (kD / 8) / kNT;     // 8
-  static constexpr int RPI = kNT / (kD / 8);          // 4
+  static constexpr int CH = kBC * (kD / 8) / NT;
+  static constexpr int RPI = NT / (kD / 8);
   op_t reg[CH];
   __device__ __forceinline__ void load(const T* tile, int rows, int64_t row_stride, int cols, int tid) {
     const int r0 = tid >> 6, cc0 = tid & 63;
@@ -97,25 +96,42 @@ struct TileFetch {
 };
 
 // ---------------------------------------------------------------------------------------------
-// forward: one workgroup = 32 query rows of one head
+// forward: one workgroup = 64 query rows of one head = 8 waves, four per 32-row block
 // ---------------------------------------------------------------------------------------------
+// A K/V tile of 32 keys is 64 KB; with 32 rows per workgroup that is 32 FLOP per byte streamed and
+// the kernel runs at the rate the L2 delivers K/V (about 225 TFLOP/s).  Two row blocks share the
+// tile here; each has its own four waves (one per 128 columns), so a SIMD holds two waves and one
+// covers the other's waits.  One K/V stage in LDS, the next tile waits in registers.
+constexpr int kFRB = 2;              // 32-row blocks per workgroup
+constexpr int kFBR = 32 * kFRB;      // query rows per workgroup
+constexpr int kFNT = kFRB * kNT;     // threads per workgroup
+struct SmemFwd512 {
+  static constexpr int ASTR = Smem512::ASTR, BSTR = Smem512::BSTR;
+  static constexpr int V_OFF = Smem512::A_ELEMS * 2;
+  static constexpr int PART_OFF = V_OFF + Smem512::B_ELEMS * 2;
+  static constexpr int BYTES = PART_OFF + kFRB * Smem512::PART_BYTES;
+};
+
 template <typename T, bool kWindowed, bool kBias, bool kDropout>
-__global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
   using Tr = Traits<T>;
   using op_t = typename Tr::op_t;
   using q4_t = typename Tr::q4_t;
-  using SM = Smem512;
+  using SM = SmemFwd512;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   T* Ks = reinterpret_cast<T*>(smem_raw);
-  T* Vs = Ks + SM::STAGES * SM::A_ELEMS;
-  float* part = reinterpret_cast<float*>(smem_raw + SM::PART_OFF);
+  T* Vs = reinterpret_cast<T*>(smem_raw + SM::V_OFF);
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rb = wave / kNW, cw = wave % kNW;             // row block, column share
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, h = blockIdx.y, mt = blockIdx.x;
+  const int z = blockIdx.z, h = blockIdx.y;
+  // (the tiles with the most visible keys of a causal mask start first)
+  const int mt = gridDim.x - 1 - blockIdx.x;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
-  if (kDropout && mt == 0 && h == 0 && z == 0 && tid == 0) {
+  float* part = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * (Smem512::PART_BYTES / 4);
+  if (kDropout && blockIdx.x == 0 && h == 0 && z == 0 && tid == 0) {
     // modules/flash/kernel/fwd_kernel.py:199-207
     uint64_t base = a.drop.offset2;
     if (a.drop.offset1_ptr) base += *a.drop.offset1_ptr;
@@ -124,7 +140,7 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
   }
 
   const SeqInfo si = get_seq(a.seq, z);
-  const int q0 = mt * kBR;
+  const int q0 = mt * kFBR;
   if (q0 >= si.seqlen_q) return;
 
   Window w{0, 0};
@@ -132,13 +148,13 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
                                   si.seqlen_q, si.seqlen_k);
   w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
   w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
-  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kBR, kBC);
+  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kFBR, kBC);
 
   const int hk = h / (a.hq / a.hk);                       // fwd_kernel.py:360
-  const int row = q0 + c;                                 // this lane's query row (the same in all waves)
+  const int row = q0 + 32 * rb + c;                       // this lane's query row (the same in the four waves of a row block)
   const bool row_ok = row < si.seqlen_q;
   const int row_c = row_ok ? row : si.seqlen_q - 1;
-  const int col0 = wave * kDW;                            // first column of this wave's share
+  const int col0 = cw * kDW;                              // first column of this wave's share
 
   T* optr = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
             (int64_t)(si.q_start + row_c) * a.so.s + col0;
@@ -153,7 +169,7 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
 #pragma unroll
         for (int g = 0; g < 4; ++g)
           if (col0 + 32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = zero4;
-      if (lse_ptr && wave == 0 && hi == 0) lse_ptr[row] = __builtin_inff();
+      if (lse_ptr && cw == 0 && hi == 0) lse_ptr[row] = __builtin_inff();
     }
     return;
   }
@@ -174,16 +190,16 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
   const T* vt = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                 (int64_t)(si.k_start + br.lo * kBC) * a.sv.s;
   int rows_left = si.seqlen_k - br.lo * kBC;      // > 0
-  TileFetch<T> kf, vf;
-  auto load_next_tile = [&]() {
+  TileFetch<T, kFNT> kf, vf;
+  auto fetch = [&]() {
     const int rows = rows_left < kBC ? rows_left : kBC;
     kf.load(kt, rows, a.sk.s, d_qk, tid);
     vf.load(vt, rows, a.sv.s, d_v, tid);
     kt += (int64_t)kBC * a.sk.s; vt += (int64_t)kBC * a.sv.s; rows_left -= kBC;
   };
-  auto store_tile = [&](int stage) {
-    kf.store(Ks + stage * SM::A_ELEMS, SM::ASTR, tid);
-    vf.store(Vs + stage * SM::B_ELEMS, SM::BSTR, tid);
+  auto publish = [&]() {
+    kf.store(Ks, SM::ASTR, tid);
+    vf.store(Vs, SM::BSTR, tid);
   };
 
   const T* bptr = nullptr;
@@ -217,20 +233,19 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
   // lane-constant part of the V^T operand address (see lds_read_tr8)
   const int v_lane = (4 * hi + (lane & 15) / 4) * SM::BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + col0;
 
-  load_next_tile();
-  store_tile(0);
+  fetch();
+  publish();
   __syncthreads();
   for (int j = br.lo; j <= br.hi; ++j) {
-    const int stage = (j - br.lo) & 1;
-    if (j < br.hi) load_next_tile();
+    if (j < br.hi) fetch();
     // this wave's share of S^T = K Q^T
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    const T* ks = Ks + stage * SM::A_ELEMS + c * SM::ASTR + col0 + hi * 8;
+    const T* ks = Ks + c * SM::ASTR + col0 + hi * 8;
 #pragma unroll
     for (int k = 0; k < kKS; ++k) s = Tr::mfma(*reinterpret_cast<const op_t*>(ks + k * 16), qreg[k], s);
-    part_write(part, wave, lane, s);
+    part_write(part, cw, lane, s);
     __syncthreads();
     s = part_sum(part, lane);
 
@@ -285,7 +300,7 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
       }
     }
     // O^T += V^T P^T on this wave's columns; P is cast to V's type (:274)
-    const T* vs = Vs + stage * SM::B_ELEMS + v_lane;
+    const T* vs = Vs + v_lane;
 #pragma unroll
     for (int t = 0; t < kBC / 16; ++t) {
       const op_t pb = pack8<T>(s, t);
@@ -293,8 +308,11 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
       for (int db = 0; db < kDB; ++db)
         o[db] = Tr::mfma(lds_read_tr8<T>(vs + t * 16 * SM::BSTR + db * 32, SM::BSTR), pb, o[db]);
     }
-    if (j < br.hi) store_tile(stage ^ 1);
-    __syncthreads();
+    __syncthreads();                 // the tile and the partial blocks have been read
+    if (j < br.hi) {
+      publish();
+      __syncthreads();
+    }
   }
 
   const float l = cross_sum(l_i);
@@ -311,7 +329,7 @@ __global__ __launch_bounds__(kNT) void fwd_d512_kernel(const FwdArgs a) {
         for (int r = 0; r < 4; ++r) t4[r] = Tr::cvt(o[db][4 * g + r] * inv);
         if (col0 + 32 * db + 8 * g + 4 * hi < d_v) *reinterpret_cast<q4_t*>(optr + 32 * db + 8 * g + 4 * hi) = t4;
       }
-    if (lse_ptr && wave == 0 && hi == 0)
+    if (lse_ptr && cw == 0 && hi == 0)
       lse_ptr[row] = alive ? (m_i * sc + fast_log2(l)) * kLn2 : __builtin_inff();   // fwd_kernel.py:610-612
   }
 }
@@ -741,13 +759,13 @@ int nseq_of(const SeqArgs& s, int batch) {
   return s.num_seqlens != 0 ? (s.num_seqlens < 0 ? -s.num_seqlens : s.num_seqlens) : batch;
 }
 
-template <auto kern, typename Args>
+template <auto kern, int NT = kNT, typename Args>
 hipError_t launch512(dim3 grid, int smem, hipStream_t stream, const Args& a) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;   // an empty tensor: nothing to write
   static std::atomic<uint64_t> lds_set{0};
   hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern), smem, lds_set);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, grid, dim3(kNT), smem, stream, a);
+  hipLaunchKernelGGL(kern, grid, dim3(NT), smem, stream, a);
   return hipGetLastError();
 }
 
@@ -765,9 +783,9 @@ hipError_t launch512(dim3 grid, int smem, hipStream_t stream, const Args& a) {
 
 template <typename T>
 hipError_t run_fwd_t(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
-  const dim3 grid((a.seq.max_seqlen_q + kBR - 1) / kBR, a.hq, nseq_of(a.seq, a.batch));
-  constexpr int smem = Smem512::PART_OFF + Smem512::PART_BYTES;
-#define FA_CALL(W, B, P) launch512<fwd_d512_kernel<T, W, B, P>>(grid, smem, s, a)
+  const dim3 grid((a.seq.max_seqlen_q + kFBR - 1) / kFBR, a.hq, nseq_of(a.seq, a.batch));
+  constexpr int smem = SmemFwd512::BYTES;
+#define FA_CALL(W, B, P) launch512<fwd_d512_kernel<T, W, B, P>, kFNT>(grid, smem, s, a)
   FA_D512_SWITCH(FA_CALL)
 #undef FA_CALL
 }
@@ -806,9 +824,10 @@ hipError_t run_fwd_d512(int dtype, const FwdArgs& a, bool windowed, bool bias, b
 }
 
 TileShape d512_tile_shape(int kernel_slot) {
-  // forward (kernel_slot < 0) and dQ: 32 queries per workgroup against 32 keys per step; dK/dV the
-  // other way round
-  return TileShape{kBR, kBC, kNW, kernel_slot < 0 ? Smem512::PART_OFF + Smem512::PART_BYTES : SmemBwd512::BYTES};
+  // forward (kernel_slot < 0): 64 queries per workgroup against 32 keys per step; dQ: 32 queries
+  // against 32 keys; dK/dV the other way round
+  if (kernel_slot < 0) return TileShape{kFBR, kBC, kFRB * kNW, SmemFwd512::BYTES};
+  return TileShape{kBR, kBC, kNW, SmemBwd512::BYTES};
 }
 
 }  // namespace fa
