@@ -349,12 +349,12 @@ struct SmemBwd512 {
   static constexpr int BYTES = PART_OFF + 2 * Smem512::PART_BYTES;
 };
 
-template <typename T>
-__device__ __forceinline__ void store_swizzled(const TileFetch<T>& f, char* tile, int tid) {
+template <typename T, int NT = kNT>
+__device__ __forceinline__ void store_swizzled(const TileFetch<T, NT>& f, char* tile, int tid) {
   const int r0 = tid >> 6, cc0 = tid & 63;
 #pragma unroll
-  for (int i = 0; i < TileFetch<T>::CH; ++i)
-    *reinterpret_cast<typename Traits<T>::op_t*>(tile + Swz<kD>::addr(r0 + i * TileFetch<T>::RPI, cc0)) = f.reg[i];
+  for (int i = 0; i < TileFetch<T, NT>::CH; ++i)
+    *reinterpret_cast<typename Traits<T>::op_t*>(tile + Swz<kD>::addr(r0 + i * TileFetch<T, NT>::RPI, cc0)) = f.reg[i];
 }
 
 // dK, dV: one workgroup = 32 keys of one kv-head; the lane's key is lane % 32 in every wave, the
@@ -560,29 +560,38 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
   }
 }
 
-// dQ and dB: one workgroup = 32 query rows of one head; the lane's query is lane % 32 in every
-// wave, the keys of a tile are spread over the accumulator elements.
+// dQ and dB: one workgroup = 64 query rows of one head = 8 waves, four per 32-row block (two row
+// blocks share the K/V tiles, two waves per SIMD, as in the forward); the lane's query is
+// lane % 32 of its row block, the keys of a tile are spread over the accumulator elements.
+struct SmemDq512 {
+  static constexpr int TILE_BYTES = SmemBwd512::TILE_BYTES;
+  static constexpr int PART_OFF = 2 * TILE_BYTES;
+  static constexpr int BYTES = PART_OFF + kFRB * 2 * Smem512::PART_BYTES;
+};
+
 template <typename T, bool kWindowed, bool kBias, bool kDropout>
-__global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(kFNT) void bwd_dq_d512_kernel(const BwdArgs a) {
   using Tr = Traits<T>;
   using op_t = typename Tr::op_t;
   using q4_t = typename Tr::q4_t;
-  using SM = SmemBwd512;
+  using SM = SmemDq512;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   char* Kb = smem_raw;
   char* Vb = smem_raw + SM::TILE_BYTES;
-  float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF);
-  float* partD = partS + Smem512::PART_BYTES / 4;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rb = wave / kNW, cw = wave % kNW;             // row block, column share
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, h = blockIdx.y, mt = blockIdx.x;
+  const int z = blockIdx.z, h = blockIdx.y;
+  const int mt = gridDim.x - 1 - blockIdx.x;              // most visible keys first (causal)
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
-  const int col0 = wave * kDW;
+  const int col0 = cw * kDW;
+  float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * 2 * (Smem512::PART_BYTES / 4);
+  float* partD = partS + Smem512::PART_BYTES / 4;
 
   const SeqInfo si = get_seq(a.seq, z);
-  const int q0 = mt * kBR;
+  const int q0 = mt * kFBR;
   if (q0 >= si.seqlen_q) return;
 
   Window w{0, 0};
@@ -590,10 +599,10 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
                                   si.seqlen_q, si.seqlen_k);
   w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
   w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
-  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kBR, kBC);
+  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kFBR, kBC);
 
   const int hk = h / (a.hq / a.hk);
-  const int row = q0 + c;
+  const int row = q0 + 32 * rb + c;
   const bool row_ok = row < si.seqlen_q;
   const int row_c = row_ok ? row : si.seqlen_q - 1;
   const int nkt = (si.seqlen_k + kBC - 1) / kBC;
@@ -602,12 +611,12 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
   const bool want_db = kBias && a.db != nullptr;
   T* dbhead = want_db ? reinterpret_cast<T*>(a.db) + (int64_t)si.batch_index * a.sdb_z + (int64_t)h * a.sdb_h : nullptr;
 
-  // dB of K tiles that are never visited is zero: wave w sweeps the rows w, w + 4, ...
+  // dB of K tiles that are never visited is zero: wave w sweeps the rows w, w + 8, ...
   auto zero_db = [&](int j_from, int j_to) {
     if (!want_db) return;
     const int c0 = j_from * kBC, c1 = j_to * kBC < si.seqlen_k ? j_to * kBC : si.seqlen_k;
     if (c0 >= c1) return;
-    for (int rr = wave; rr < kBR; rr += kNW) {
+    for (int rr = wave; rr < kFBR; rr += kFRB * kNW) {
       const int m = q0 + rr;
       if (m >= si.seqlen_q) break;
       T* rowp = dbhead + (int64_t)m * a.sdb_m;
@@ -665,7 +674,7 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
     const T* vt = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                   (int64_t)(si.k_start + br.lo * kBC) * a.sv.s;
     int rows_left = si.seqlen_k - br.lo * kBC;      // > 0
-    TileFetch<T> kf, vf;
+    TileFetch<T, kFNT> kf, vf;
     auto fetch = [&]() {
       const int rows = rows_left < kBC ? rows_left : kBC;
       kf.load(kt, rows, a.sk.s, d_qk, tid);
@@ -673,8 +682,8 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
       kt += (int64_t)kBC * a.sk.s; vt += (int64_t)kBC * a.sv.s; rows_left -= kBC;
     };
     auto publish = [&]() {
-      store_swizzled<T>(kf, Kb, tid);
-      store_swizzled<T>(vf, Vb, tid);
+      store_swizzled<T, kFNT>(kf, Kb, tid);
+      store_swizzled<T, kFNT>(vf, Vb, tid);
     };
 
     fetch();
@@ -688,11 +697,11 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
       for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
 #pragma unroll
       for (int k = 0; k < kKS; ++k) {
-        s = Tr::mfma(swz_read_row<T, kD>(Kb, row_a, wave * kKS + k, 0), qreg[k], s);
-        dp = Tr::mfma(swz_read_row<T, kD>(Vb, row_a, wave * kKS + k, 0), doreg[k], dp);
+        s = Tr::mfma(swz_read_row<T, kD>(Kb, row_a, cw * kKS + k, 0), qreg[k], s);
+        dp = Tr::mfma(swz_read_row<T, kD>(Vb, row_a, cw * kKS + k, 0), doreg[k], dp);
       }
-      part_write(partS, wave, lane, s);
-      part_write(partD, wave, lane, dp);
+      part_write(partS, cw, lane, s);
+      part_write(partD, cw, lane, dp);
       __syncthreads();
       s = part_sum(partS, lane);
       dp = part_sum(partD, lane);
@@ -721,7 +730,7 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
           if (kDropout) dpv = ((keep >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
           const float dsv = p * (dpv - d_row);
           dp[i] = dsv;
-          if (want_db && wave == 0 && row_ok && n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);   // :200-204
+          if (want_db && cw == 0 && row_ok && n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);   // :200-204
         }
       }
       // dQ^T += K^T dS^T on this wave's columns
@@ -730,7 +739,7 @@ __global__ __launch_bounds__(kNT) void bwd_dq_d512_kernel(const BwdArgs a) {
         const op_t sb = pack8<T>(dp, t);      // ds cast to K's type
 #pragma unroll
         for (int db = 0; db < kDB; ++db)
-          dq[db] = Tr::mfma(swz_read_tr<T, kD>(Kb, tr_a0, tr_a1, t, wave * kDB + db), sb, dq[db]);
+          dq[db] = Tr::mfma(swz_read_tr<T, kD>(Kb, tr_a0, tr_a1, t, cw * kDB + db), sb, dq[db]);
       }
       __syncthreads();                 // the tile and the partial blocks have been read
       if (j < br.hi) {
@@ -800,8 +809,8 @@ hipError_t run_bwd_t(int kernel_slot, const BwdArgs& a, bool windowed, bool bias
 #undef FA_CALL
   }
   if (kernel_slot == 2) {
-    const dim3 grid((a.seq.max_seqlen_q + kBR - 1) / kBR, a.hq, nseq);
-#define FA_CALL(W, B, P) launch512<bwd_dq_d512_kernel<T, W, B, P>>(grid, SmemBwd512::BYTES, s, a)
+    const dim3 grid((a.seq.max_seqlen_q + kFBR - 1) / kFBR, a.hq, nseq);
+#define FA_CALL(W, B, P) launch512<bwd_dq_d512_kernel<T, W, B, P>, kFNT>(grid, SmemDq512::BYTES, s, a)
     FA_D512_SWITCH(FA_CALL)
 #undef FA_CALL
   }
@@ -824,10 +833,11 @@ hipError_t run_fwd_d512(int dtype, const FwdArgs& a, bool windowed, bool bias, b
 }
 
 TileShape d512_tile_shape(int kernel_slot) {
-  // forward (kernel_slot < 0): 64 queries per workgroup against 32 keys per step; dQ: 32 queries
-  // against 32 keys; dK/dV the other way round
+  // forward (kernel_slot < 0) and dQ: 64 queries per workgroup against 32 keys per step; dK/dV: 32
+  // keys per workgroup against 32 queries per step
   if (kernel_slot < 0) return TileShape{kFBR, kBC, kFRB * kNW, SmemFwd512::BYTES};
-  return TileShape{kBR, kBC, kNW, SmemBwd512::BYTES};
+  if (kernel_slot == 2) return TileShape{kFBR, kBC, kFRB * kNW, SmemDq512::BYTES};
+  return TileShape{kBC, kBR, kNW, SmemBwd512::BYTES};
 }
 
 }  // namespace fa
