@@ -69,6 +69,36 @@ __device__ __forceinline__ f32x16 part_sum(const float* area, int lane) {
   return x;
 }
 
+// Backward: the element work on a summed block needs no row reduction, so it is split as well:
+// wave g adds only elements 4 g .. 4 g + 3 of every lane (a quarter of each partial block), does the
+// exponentials, mask, dropout and dS for those, and hands the two results to all waves as 16-bit
+// MFMA operand pieces (8 bytes per lane and quarter); slots 2 t and 2 t + 1 form the operand of
+// k-step t.
+__device__ __forceinline__ f32x4 part_sum_quarter(const float* area, int g, int lane) {
+  f32x4 acc = *reinterpret_cast<const f32x4*>(area + (g * 64 + lane) * 4);
+#pragma unroll
+  for (int w = 1; w < kNW; ++w) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(area + ((w * 4 + g) * 64 + lane) * 4);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] += t[r];
+  }
+  return acc;
+}
+template <typename T>
+__device__ __forceinline__ void opnd_write(char* area, int g, int lane, const f32x4& x) {
+  typename Traits<T>::q4_t q;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) q[r] = Traits<T>::cvt(x[r]);
+  *reinterpret_cast<typename Traits<T>::q4_t*>(area + (g * 64 + lane) * 8) = q;
+}
+template <typename T>
+__device__ __forceinline__ typename Traits<T>::op_t opnd_read(const char* area, int t, int lane) {
+  const auto lo = *reinterpret_cast<const typename Traits<T>::q4_t*>(area + ((2 * t) * 64 + lane) * 8);
+  const auto hi = *reinterpret_cast<const typename Traits<T>::q4_t*>(area + ((2 * t + 1) * 64 + lane) * 8);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+constexpr int kOpndBytes = 4 * 64 * 8;     // one operand block: 4 quarters x 64 lanes x 8 bytes
+
 // A tile of kBC rows x 512 columns, global -> registers -> LDS by the whole workgroup of NT threads:
 // a wave instruction covers one row (64 pieces of 16 bytes), a thread holds its pieces NT / 64
 // rows apart.  The buffer descriptor bounds the tile to its valid rows and columns; what lies
@@ -346,7 +376,8 @@ struct SmemBwd512 {
   static constexpr int TILE_BYTES = kBC * kD * 2;
   static constexpr int STAT_OFF = 2 * TILE_BYTES;
   static constexpr int PART_OFF = STAT_OFF + 2 * kBC * 4;
-  static constexpr int BYTES = PART_OFF + 2 * Smem512::PART_BYTES;
+  static constexpr int OPND_OFF = PART_OFF + 2 * Smem512::PART_BYTES;     // P and dS operand pieces
+  static constexpr int BYTES = OPND_OFF + 2 * kOpndBytes;
 };
 
 template <typename T, int NT = kNT>
@@ -372,6 +403,8 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
   float* Ds = Ls + kBC;
   float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF);
   float* partD = partS + Smem512::PART_BYTES / 4;
+  char* opP = smem_raw + SM::OPND_OFF;
+  char* opS = opP + kOpndBytes;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -483,8 +516,9 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
       part_write(partS, wave, lane, s);
       part_write(partD, wave, lane, dp);
       __syncthreads();
-      s = part_sum(partS, lane);
-      dp = part_sum(partD, lane);
+      // this wave's quarter of the elements: queries m0 + 8 wave + 4 hi + r
+      const f32x4 s4 = part_sum_quarter(partS, wave, lane);
+      const f32x4 dp4 = part_sum_quarter(partD, wave, lane);
 
       DropoutState dst{};
       if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
@@ -493,42 +527,41 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
         bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)hq * a.sb_h +
                (int64_t)key_c * a.sb_n;
       const bool masked = !br.is_full(e);
-      const unsigned q_d = q_none ? 0x40000000u : (unsigned)(m0 + 4 * hi - q_lo);
-      f32x16 pd;      // p as the dV GEMM sees it (dropped and scaled)
+      const unsigned q_d = q_none ? 0x40000000u : (unsigned)(m0 + 8 * wave + 4 * hi - q_lo);
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(Ls + 8 * wave + 4 * hi);
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(Ds + 8 * wave + 4 * hi);
+      f32x4 pd, dsv;      // p as the dV GEMM sees it (dropped and scaled), dS
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(Ls + 8 * g + 4 * hi);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(Ds + 8 * g + 4 * hi);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = 4 * g + r;
-          const int m = m0 + 8 * g + 4 * hi + r;
-          // p = exp2(s c + bias log2e - L log2e) (bwd_inner_dk_dv.py:187-188)
-          float x = s[i] * qk_scale - l4[r];
-          if (kBias) {
-            const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
-            x = __builtin_fmaf((float)bptr[(int64_t)mm * a.sb_m], kLog2e, s[i] * qk_scale) - l4[r];
-          }
-          if (masked) {
-            const bool vis = q_d + (unsigned)(8 * g + r) <= q_rng;
-            x = vis ? x : -__builtin_inff();
-          }
-          const float p = fast_exp2(x);
-          float pv = p, dpv = dp[i];
-          if (kDropout) {
-            const bool keep = dropout_keep1(dst, m, key);
-            pv = keep ? p * dst.scale : 0.f;                       // :200-201
-            dpv = keep ? dpv * dst.scale : 0.f;                    // :239-240
-          }
-          pd[i] = pv;
-          dp[i] = p * (dpv - d4[r]);                               // ds uses the undropped p (:242)
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + 8 * wave + 4 * hi + r;
+        // p = exp2(s c + bias log2e - L log2e) (bwd_inner_dk_dv.py:187-188)
+        float x = s4[r] * qk_scale - l4[r];
+        if (kBias) {
+          const int mm = m < si.seqlen_q ? m : si.seqlen_q - 1;
+          x = __builtin_fmaf((float)bptr[(int64_t)mm * a.sb_m], kLog2e, s4[r] * qk_scale) - l4[r];
         }
+        if (masked) {
+          const bool vis = q_d + (unsigned)r <= q_rng;
+          x = vis ? x : -__builtin_inff();
+        }
+        const float p = fast_exp2(x);
+        float pv = p, dpv = dp4[r];
+        if (kDropout) {
+          const bool keep = dropout_keep1(dst, m, key);
+          pv = keep ? p * dst.scale : 0.f;                       // :200-201
+          dpv = keep ? dpv * dst.scale : 0.f;                    // :239-240
+        }
+        pd[r] = pv;
+        dsv[r] = p * (dpv - d4[r]);                              // ds uses the undropped p (:242)
       }
+      opnd_write<T>(opP, wave, lane, pd);       // p cast to dO's type (composed_tensors.py:191-193)
+      opnd_write<T>(opS, wave, lane, dsv);
+      __syncthreads();
       // dV^T += dO^T P and dK^T += Q^T dS on this wave's columns
 #pragma unroll
       for (int t = 0; t < kBC / 16; ++t) {
-        const op_t pb = pack8<T>(pd, t);      // p cast to dO's type (composed_tensors.py:191-193)
-        const op_t sb = pack8<T>(dp, t);
+        const op_t pb = opnd_read<T>(opP, t, lane);
+        const op_t sb = opnd_read<T>(opS, t, lane);
 #pragma unroll
         for (int db = 0; db < kDB; ++db) {
           dv[db] = Tr::mfma(swz_read_tr<T, kD>(dOb, tr_a0, tr_a1, t, wave * kDB + db), pb, dv[db]);
@@ -566,7 +599,8 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
 struct SmemDq512 {
   static constexpr int TILE_BYTES = SmemBwd512::TILE_BYTES;
   static constexpr int PART_OFF = 2 * TILE_BYTES;
-  static constexpr int BYTES = PART_OFF + kFRB * 2 * Smem512::PART_BYTES;
+  static constexpr int OPND_OFF = PART_OFF + kFRB * 2 * Smem512::PART_BYTES;   // dS operand pieces per row block
+  static constexpr int BYTES = OPND_OFF + kFRB * kOpndBytes;
 };
 
 template <typename T, bool kWindowed, bool kBias, bool kDropout>
@@ -589,6 +623,7 @@ __global__ __launch_bounds__(kFNT) void bwd_dq_d512_kernel(const BwdArgs a) {
   const int col0 = cw * kDW;
   float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * 2 * (Smem512::PART_BYTES / 4);
   float* partD = partS + Smem512::PART_BYTES / 4;
+  char* opS = smem_raw + SM::OPND_OFF + rb * kOpndBytes;
 
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * kFBR;
@@ -703,40 +738,40 @@ __global__ __launch_bounds__(kFNT) void bwd_dq_d512_kernel(const BwdArgs a) {
       part_write(partS, cw, lane, s);
       part_write(partD, cw, lane, dp);
       __syncthreads();
-      s = part_sum(partS, lane);
-      dp = part_sum(partD, lane);
+      // this wave's quarter of its row block's elements: keys j kBC + 8 cw + 4 hi + r
+      const f32x4 s4 = part_sum_quarter(partS, cw, lane);
+      const f32x4 dp4 = part_sum_quarter(partD, cw, lane);
 
       const bool masked = !br.is_full(j);
-      const unsigned m_d = m_none ? 0x40000000u : (unsigned)(j * kBC + 4 * hi - m_lo);
+      const unsigned m_d = m_none ? 0x40000000u : (unsigned)(j * kBC + 8 * cw + 4 * hi - m_lo);
+      uint32_t keep = 0xfu;
+      if (kDropout) keep = dropout_keep4(dst, row, j * kBC + 8 * cw + 4 * hi);
+      f32x4 dsv4;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint32_t keep = 0xfu;
-        if (kDropout) keep = dropout_keep4(dst, row, j * kBC + 8 * g + 4 * hi);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = 4 * g + r;
-          const int n = j * kBC + 8 * g + 4 * hi + r;
-          float x = s[i] * qk_scale - l_row;
-          if (kBias) {
-            const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
-            x = __builtin_fmaf((float)bptr[(int64_t)nn * a.sb_n], kLog2e, s[i] * qk_scale) - l_row;
-          }
-          if (masked) {
-            const bool vis = m_d + (unsigned)(8 * g + r) <= m_rng;
-            x = vis ? x : -__builtin_inff();
-          }
-          const float p = fast_exp2(x);
-          float dpv = dp[i];
-          if (kDropout) dpv = ((keep >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
-          const float dsv = p * (dpv - d_row);
-          dp[i] = dsv;
-          if (want_db && cw == 0 && row_ok && n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);   // :200-204
+      for (int r = 0; r < 4; ++r) {
+        const int n = j * kBC + 8 * cw + 4 * hi + r;
+        float x = s4[r] * qk_scale - l_row;
+        if (kBias) {
+          const int nn = n < si.seqlen_k ? n : si.seqlen_k - 1;
+          x = __builtin_fmaf((float)bptr[(int64_t)nn * a.sb_n], kLog2e, s4[r] * qk_scale) - l_row;
         }
+        if (masked) {
+          const bool vis = m_d + (unsigned)r <= m_rng;
+          x = vis ? x : -__builtin_inff();
+        }
+        const float p = fast_exp2(x);
+        float dpv = dp4[r];
+        if (kDropout) dpv = ((keep >> r) & 1u) ? dpv * dst.scale : 0.f;   // bwd_inner_dq.py:176-185
+        const float dsv = p * (dpv - d_row);
+        dsv4[r] = dsv;
+        if (want_db && row_ok && n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);   // :200-204
       }
+      opnd_write<T>(opS, cw, lane, dsv4);       // ds cast to K's type
+      __syncthreads();
       // dQ^T += K^T dS^T on this wave's columns
 #pragma unroll
       for (int t = 0; t < kBC / 16; ++t) {
-        const op_t sb = pack8<T>(dp, t);      // ds cast to K's type
+        const op_t sb = opnd_read<T>(opS, t, lane);
 #pragma unroll
         for (int db = 0; db < kDB; ++db)
           dq[db] = Tr::mfma(swz_read_tr<T, kD>(Kb, tr_a0, tr_a1, t, cw * kDB + db), sb, dq[db]);
