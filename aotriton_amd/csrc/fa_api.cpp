@@ -316,7 +316,8 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
-  if (dtype == FA_DTYPE_FLOAT32) return fa::run_fwd_valu(dtype, d, a, stream);
+  if (dtype == FA_DTYPE_FLOAT32)
+    return d <= 256 ? fa::run_fwd_f32(d, a, s.windowed, s.bias, s.dropout, stream) : fa::run_fwd_valu(dtype, d, a, stream);
   if (d > 256) return fa::run_fwd_d512(dtype, a, s.windowed, s.bias, s.dropout, stream);
   const bool padded = a.head_dim != d || a.head_dim_v != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
@@ -409,7 +410,8 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   if (e != FA_SUCCESS) return e;
   // the vector-ALU kernels (fp32) and the split-head-dim kernels (above 256): 32 rows per workgroup, 3-D grid
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;
-  const fa::TileShape t = params->Q.dtype == FA_DTYPE_FLOAT32 ? fa::TileShape{32, 1, 4, 0}
+  const fa::TileShape t = params->Q.dtype == FA_DTYPE_FLOAT32
+                              ? (s.d <= 256 ? fa::f32_tile_shape(s.d, -1) : fa::TileShape{32, 1, 4, 0})
                           : s.d > 256 ? fa::d512_tile_shape(-1)
                                       : fa::fwd_tile_shape(params->Q.dtype, s.d, s.windowed);
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
@@ -448,7 +450,9 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
   if (valu && kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
   const bool split_d = params->Q.dtype != FA_DTYPE_FLOAT32 && s.d > 256 && kernel_slot != 0;
-  const fa::TileShape t = split_d ? fa::d512_tile_shape(kernel_slot)
+  const bool f32_mfma = params->Q.dtype == FA_DTYPE_FLOAT32 && s.d <= 256 && kernel_slot != 0;
+  const fa::TileShape t = f32_mfma ? fa::f32_tile_shape(s.d, kernel_slot)
+                          : split_d ? fa::d512_tile_shape(kernel_slot)
                           : valu  ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
                                   : fa::bwd_tile_shape(params->Q.dtype, s.d, s.windowed, kernel_slot);
   const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
@@ -643,18 +647,22 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       }
     }
     a.delta = static_cast<float*>(delta.ptr);
-    const bool f32 = dt == FA_DTYPE_FLOAT32;      // vector-ALU kernels
-    const bool big = !f32 && s.d > 256;           // head dim split over the waves; delta from the vector-ALU kernel
+    const bool f32 = dt == FA_DTYPE_FLOAT32;      // fp32 MFMA kernels up to head dim 256, vector-ALU kernels above
+    const bool big = !f32 && s.d > 256;           // head dim split over the waves
+    // (delta of both comes from the vector-ALU kernel)
     if (kernel_slot < 0 || kernel_slot == 0)
       err = f32 || big ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
-    if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 1))
-      err = f32   ? fa::run_bwd_valu(dt, s.d, 1, a, stream)
-            : big ? fa::run_bwd_d512(dt, 1, a, s.windowed, s.bias, s.dropout, stream)
-                  : fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
-    if (err == hipSuccess && (kernel_slot < 0 || kernel_slot == 2))
-      err = f32   ? fa::run_bwd_valu(dt, s.d, 2, a, stream)
-            : big ? fa::run_bwd_d512(dt, 2, a, s.windowed, s.bias, s.dropout, stream)
-                  : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+    for (int slot = 1; slot <= 2 && err == hipSuccess; ++slot) {
+      if (kernel_slot >= 0 && kernel_slot != slot) continue;
+      if (f32)
+        err = s.d <= 256 ? fa::run_bwd_f32(s.d, slot, a, s.windowed, s.bias, s.dropout, stream)
+                         : fa::run_bwd_valu(dt, s.d, slot, a, stream);
+      else if (big)
+        err = fa::run_bwd_d512(dt, slot, a, s.windowed, s.bias, s.dropout, stream);
+      else
+        err = slot == 1 ? fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream)
+                        : fa::run_bwd_dq(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+    }
     if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);   // attn_bwd.cc:157
   } else {
     a.delta = nullptr;

@@ -38,6 +38,13 @@ hipError_t run_bwd_d512(int dtype, int kernel_slot, const BwdArgs& a, bool windo
                         hipStream_t s);
 TileShape d512_tile_shape(int kernel_slot);
 
+// MFMA kernels for fp32 tensors at head dims up to 256 (compiled for 128 and 256 columns, the head
+// dim split over the waves of a workgroup).  kernel_slot of the backward: 1 dK/dV, 2 dQ and dB.
+hipError_t run_fwd_f32(int head_dim, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
+hipError_t run_bwd_f32(int head_dim, int kernel_slot, const BwdArgs& a, bool windowed, bool bias, bool dropout,
+                       hipStream_t s);
+TileShape f32_tile_shape(int head_dim, int kernel_slot);
+
 // Vector-ALU kernels (no MFMA): fp32 tensors at any head dim, every type at head dim 512.
 // head_dim is the compiled one (64, 128, 256, 512).  kernel_slot of the backward: 0 delta,
 // 1 dK/dV, 2 dQ and dB.
