@@ -120,7 +120,7 @@ def test_validate_fwd_error_contract():
         pb, kb = _fwd_params(D=bad)
         assert validate_fwd(pb, 3) == E.hipErrorNotSupported
     p3, k3 = _fwd_params(dtype=torch.float32)
-    assert validate_fwd(p3, 3) == E.hipSuccess                                 # fp32: vector-ALU kernels
+    assert validate_fwd(p3, 3) == E.hipSuccess                                 # fp32: fp32 MFMA kernels
     p4, k4 = _fwd_params(Hq=5, Hk=2)
     assert validate_fwd(p4, 3) == E.hipErrorInvalidValue                       # heads not divisible
     p.Q = T4(0, [0] * 4, [0] * 4, DType.kBFloat16)
