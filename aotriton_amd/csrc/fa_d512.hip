@@ -317,10 +317,12 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
       rs += s[i];                       // the row sum is over the fp32, undropped p (:213-214)
     }
     l_i = l_i * alpha + rs;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // some row of the wave moved its maximum
 #pragma unroll
-    for (int db = 0; db < kDB; ++db)
+      for (int db = 0; db < kDB; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
     if (kDropout) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {

@@ -94,7 +94,7 @@ def main():
                          'written) so that FETCH_SIZE / WRITE_SIZE counters can be scaled')
     ap.add_argument('--tile-entry', default=None, metavar='D,causal,dtype',
                     help='run the forward, dK/dV and dQ kernels of one tile-table entry a few times and print their '
-                         'times (for profiler runs), e.g. 64,1,bf16: B = 4, H = 4096 / D, S = 4096')
+                         'times (for profiler runs), e.g. 64,1,bf16: B = 4, H = 4096 / D, S = 4096; D up to 512, dtype bf16, fp16 or fp32')
     ap.add_argument('--mfma-peak', action='store_true',
                     help='only measure what the matrix pipe sustains (register-only MFMA loop, constant '
                          'and random operands) and print that as one JSON line')
@@ -149,7 +149,7 @@ def main():
     if args.tile_entry:
         d_s, c_s, t_s = args.tile_entry.split(',')
         D, causal = int(d_s), bool(int(c_s))
-        dtype = {'bf16': torch.bfloat16, 'fp16': torch.float16}[t_s]
+        dtype = {'bf16': torch.bfloat16, 'fp16': torch.float16, 'fp32': torch.float32}[t_s]
         B, S = 4, 4096
         H = 4096 // D
         g = torch.Generator(device=dev).manual_seed(1234)
