@@ -649,10 +649,16 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     a.delta = static_cast<float*>(delta.ptr);
     const bool f32 = dt == FA_DTYPE_FLOAT32;      // fp32 MFMA kernels up to head dim 256, vector-ALU kernels above
     const bool big = !f32 && s.d > 256;           // head dim split over the waves
-    // (delta of both comes from the vector-ALU kernel)
-    if (kernel_slot < 0 || kernel_slot == 0)
-      err = f32 || big ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
-    for (int slot = 1; slot <= 2 && err == hipSuccess; ++slot) {
+    // fp32 and the head dims above 256 take delta from the vector-ALU kernel.  The dQ kernel of the
+    // 16-bit types up to head dim 256 computes delta from the O and dO rows it holds and writes it
+    // out; the dK/dV kernel runs after it and reads it, so the whole backward is two launches
+    // (kernel_slot 0 still launches the preprocess kernel on its own).
+    const bool delta_launch = f32 || big;
+    if (kernel_slot == 0 || (kernel_slot < 0 && delta_launch))
+      err = delta_launch ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
+    const int order[2] = {delta_launch ? 1 : 2, delta_launch ? 2 : 1};
+    for (int i = 0; i < 2 && err == hipSuccess; ++i) {
+      const int slot = order[i];
       if (kernel_slot >= 0 && kernel_slot != slot) continue;
       if (f32)
         err = s.d <= 256 ? fa::run_bwd_f32(s.d, slot, a, s.windowed, s.bias, s.dropout, stream)

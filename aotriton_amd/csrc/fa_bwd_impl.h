@@ -762,7 +762,11 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 // ---------------------------------------------------------------------------
 // dQ (+dB) work item
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta, bool kPad>
+// kInlineDelta: delta = rowsum(O dO) of the item's rows is computed here, from the rows the lanes
+// load anyway (dO) and their O rows, instead of being read.  kStoreDelta: it is also written out:
+// the split backward has no preprocess launch, the dK/dV kernel runs after this one and reads it.
+template <typename T, int D, int NW, int BN, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta, bool kPad,
+          bool kStoreDelta = false>
 __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int mt, const int z,
                                         char* smem_raw) {
   using Tr = Traits<T>;
@@ -846,6 +850,24 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         for (int g = 0; g < 4; ++g)
           if (32 * db + 8 * g + 4 * hi < d_qk) *reinterpret_cast<q4_t*>(dqptr + 32 * db + 8 * g + 4 * hi) = zero4;
     }
+    if (kStoreDelta) {
+      // no key sees these rows and nobody reads their delta; it is written all the same, as the
+      // preprocess kernel would (bwd_preprocess.py:28-250)
+      const T* optr = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z +
+                      (int64_t)h * a.so.h + (int64_t)(si.q_start + row_c) * a.so.s;
+      const T* doptr = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
+                       (int64_t)h * a.sdo.h + (int64_t)(si.q_start + row_c) * a.sdo.s;
+      float acc = 0.f;
+      for (int k = 0; k < KS; ++k) {
+        if (16 * k + 8 * hi >= d_v) continue;
+        const op_t o8 = *reinterpret_cast<const op_t*>(optr + 16 * k + 8 * hi);
+        const op_t d8 = *reinterpret_cast<const op_t*>(doptr + 16 * k + 8 * hi);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)o8[e] * (float)d8[e];
+      }
+      acc = cross_sum(acc);
+      if (row_ok && hi == 0) a.delta[lse_offset(si, h, a.hq) + row] = acc;
+    }
     zero_db(0, nkt);
     return;
   }
@@ -877,6 +899,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       for (int e = 0; e < 8; ++e) acc += (float)o8[e] * (float)doreg[k][e];
     }
     d_row = cross_sum(acc);
+    if (kStoreDelta && row_ok && hi == 0) a.delta[lo] = d_row;
   } else {
     d_row = a.delta[lo];
   }
@@ -896,7 +919,7 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
   // Without dropout (the mask and the scale come between dP and the subtraction) dP starts at
   // -delta.  Not in the dQ kernel at D = 64: with 128-key tiles its register allocation gets
   // worse with the extra tuple (20-50 % slower); the single-launch kernel at D = 64 gains.
-  constexpr bool kFoldDelta = !kDropout && (D >= 128 || kInlineDelta);
+  constexpr bool kFoldDelta = !kDropout && (D >= 128 || (kInlineDelta && !kStoreDelta));
   f32x16 negd16;      // -delta of this lane's query in every element: the initial value of dP
 #pragma unroll
   for (int i = 0; i < 16; ++i) negd16[i] = -d_row;
@@ -1322,7 +1345,7 @@ void bwd_dq_kernel(const BwdArgs a) {
     const int mt = a.num_m_tiles - 1 - gr / a.zh_group;
     int z, h;
     split_zh(zh, a.num_zh / a.hq, a.hq / a.hk, z, h);
-    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, false, kPad>(a, h, mt, z, smem_raw);
+    dq_item<T, D, NW, BN, kWindowed, kBias, kDropout, true, kPad, true>(a, h, mt, z, smem_raw);
     __syncthreads();     // the next item reuses the LDS stages
   }
 }

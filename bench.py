@@ -291,19 +291,21 @@ def main():
     dom_r, dom_fl = kernels[dom]
     dom_ms = dom_r['mean']
     # the backward as a whole in the reference's convention (5 GEMMs of algorithmic work, 7 executed)
-    bwd_kernels_ms = r_pre['mean'] + r_dkdv['mean'] + r_dq['mean']
+    # (the dQ kernel computes delta itself and hands it to the dK/dV kernel: two launches)
+    bwd_kernels_ms = r_dkdv['mean'] + r_dq['mean']
     elem = 2 * B * H * S * D                                   # bytes of one bf16 activation tensor
     algorithmic_bytes = {'fwd_kernel': 4 * elem + 4 * B * H * S,            # Q, K, V in, O out, LSE out
                          'bwd_dkdv_kernel': 6 * elem + 8 * B * H * S,       # Q, K, V, dO in, dK, dV out, LSE, delta in
-                         'bwd_dq_kernel': 5 * elem + 8 * B * H * S}         # Q, K, V, dO in, dQ out, LSE, delta in
+                         'bwd_dq_kernel': 6 * elem + 8 * B * H * S}         # Q, K, V, O, dO in, dQ out, LSE in, delta out
     roofline = {'bound': 'mfma', 'kernel': dom, 'achieved': tf(dom_fl, dom_ms), 'peak': PEAK_BF16_TFLOPS,
                 'unit': 'TFLOP/s', 'frac': tf(dom_fl, dom_ms) / PEAK_BF16_TFLOPS,
                 'traffic': hbm_bytes_from_profile(dom), 'algorithmic_bytes': algorithmic_bytes[dom],
                 'avg_ms': dom_ms, 'median_ms': dom_r['median'], 'flop_per_launch': dom_fl,
                 'frac_ref_convention': tf(f_bwd, bwd_kernels_ms) / PEAK_BF16_TFLOPS,
                 'frac_ref_convention_note': 'whole split backward: 2.5 x forward FLOP (5 GEMMs) over the summed '
-                                            'mean durations of its three kernels; frac counts the GEMMs the '
-                                            'dominant kernel executes'}
+                                            'mean durations of its two kernels (dQ, which also computes '
+                                            'delta, then dK/dV); frac counts the GEMMs the dominant kernel '
+                                            'executes'}
 
     out = {
         'metric': 'attn fwd/bwd TFLOPS and % bf16 MFMA peak, B4 H32 S4096 D128 causal, 1 GPU',
@@ -317,8 +319,8 @@ def main():
         'timing': 'per launch: 512 MiB zeroed before it, warm-up >= 25 ms, >= 100 ms of launches, HIP events, '
                   'median (p20, p80); value/ms_per_step: K back-to-back steps between synchronisations',
         'fwd': row(f_fwd, r_fwd),
-        'bwd_split': row(f_bwd, r_split, {'kernels_ms': {'bwd_preprocess': r_pre['median'], 'bwd_dkdv': r_dkdv['median'],
-                                                         'bwd_dq': r_dq['median']}}),
+        'bwd_split': row(f_bwd, r_split, {'kernels_ms': {'bwd_dq_with_delta': r_dq['median'], 'bwd_dkdv': r_dkdv['median'],
+                                                         'bwd_preprocess_standalone_not_launched': r_pre['median']}}),
         'bwd_fused': row(f_bwd, r_fused),
         'roofline': roofline,
     }
