@@ -106,8 +106,10 @@ typedef struct fa_lazy_tensor4 {
 } fa_lazy_tensor4;
 
 /* attn_options, include/aotriton/flash.h:38-41.
- * Backward backends: 0 = split (preprocess + dK/dV + dQ), 1 = fused single
- * launch (modules/flash/aot/__init__.py:83-85).  Index 2 (prebuilt assembly
+ * Backward backends: 0 = split (the reference's preprocess + dK/dV + dQ; here dQ,
+ * which also computes delta and writes it to params->D, then dK/dV; fp32 tensors and
+ * head dims above 256 launch a delta kernel first), 1 = fused single launch
+ * (modules/flash/aot/__init__.py:83-85).  Index 2 (prebuilt assembly
  * backend of the reference) does not exist here and is rejected with
  * FA_ERROR_PEER_ACCESS_UNSUPPORTED.  Forward has backend 0 only. */
 typedef struct fa_options {
@@ -274,8 +276,9 @@ FA_API int fa_v2_attn_bwd_compact_varlen(
 FA_API int fa_attn_bwd_noalloc(const fa_bwd_params* params, int32_t params_version,
                                void* hip_stream);
 
-/* One kernel of the backward only: kernel_slot 0 = delta (bwd_preprocess), 1 = dK/dV,
- * 2 = dQ, 3 = fused.  Slots 0-2 need an eager delta buffer in params->D.  Stands in
+/* One kernel of the backward only: kernel_slot 0 = delta (bwd_preprocess), 1 = dK/dV
+ * (reads delta), 2 = dQ (16-bit types up to head dim 256: computes delta and writes it;
+ * otherwise reads it), 3 = fused.  Slots 0-2 need an eager delta buffer in params->D.  Stands in
  * for the per-kernel selection of the reference's tuning interface
  * (attn_options::KernelSlot, include/aotriton/flash.h:46-60; include/aotriton/cpp_tune.h)
  * and is what the benchmark uses to time kernels one at a time. */
