@@ -417,9 +417,14 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
   out->lds_bytes = t.lds_bytes;
   if (valu) {
-    out->grid[0] = (s.max_sq + t.block_m - 1) / t.block_m;
-    out->grid[1] = s.hq;
-    out->grid[2] = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+    const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
+    const int mt = (s.max_sq + t.block_m - 1) / t.block_m;
+    if (params->Q.dtype == FA_DTYPE_FLOAT32 && s.d > 256) {      // vector-ALU kernels: 3-D grid
+      out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz;
+    } else {      // one workgroup per tile, the tiles of a kv-head's group back to back on one XCD
+      out->grid[0] = fa::kNumXcd * ((nz * s.hk + fa::kNumXcd - 1) / fa::kNumXcd) * (s.hq / s.hk) * mt;
+      out->grid[1] = 1; out->grid[2] = 1;
+    }
   } else {
     const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
     const int zh_per_xcd = (nz * s.hq + fa::kNumXcd - 1) / fa::kNumXcd;
@@ -474,7 +479,9 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   const int ratio = s.hq / s.hk;
   out->grid[1] = 1;
   out->grid[2] = 1;
-  if (valu) {
+  if (f32_mfma || split_d) {      // one workgroup per tile, the tiles of a kv-head back to back on one XCD
+    out->grid[0] = fa::kNumXcd * ((nz * s.hk + fa::kNumXcd - 1) / fa::kNumXcd) * (kernel_slot == 1 ? nt : ratio * mt);
+  } else if (valu) {
     out->grid[0] = kernel_slot == 1 ? nt : mt;
     out->grid[1] = kernel_slot == 1 ? s.hk : s.hq;
     out->grid[2] = nz;

@@ -156,12 +156,16 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb = wave / kNW, cw = wave % kNW;             // row block, column share
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, h = blockIdx.y;
-  // (the tiles with the most visible keys of a causal mask start first)
-  const int mt = gridDim.x - 1 - blockIdx.x;
+  // one workgroup per (sequence, q-head, Q tile): the tiles of a kv-head's group back to back on one
+  // XCD, most visible keys (causal) first
+  const int nmt = (a.seq.max_seqlen_q + kFBR - 1) / kFBR, group = a.hq / a.hk;
+  int pair, r_item;
+  if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, group * nmt, pair, r_item)) return;
+  const int z = pair / a.hk, h = (pair % a.hk) * group + r_item % group;
+  const int mt = nmt - 1 - r_item / group;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   float* part = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * (Smem512::PART_BYTES / 4);
-  if (kDropout && blockIdx.x == 0 && h == 0 && z == 0 && tid == 0) {
+  if (kDropout && blockIdx.x == 0 && tid == 0) {
     // modules/flash/kernel/fwd_kernel.py:199-207
     uint64_t base = a.drop.offset2;
     if (a.drop.offset1_ptr) base += *a.drop.offset1_ptr;
@@ -411,7 +415,11 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, hk = blockIdx.y, nt = blockIdx.x;
+  // one workgroup per (sequence, kv-head, key block): the key blocks of a kv-head back to back on
+  // one XCD, those that the most queries see (causal) first
+  int pair, nt;
+  if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, (a.seq.max_seqlen_k + kBR - 1) / kBR, pair, nt)) return;
+  const int z = pair / a.hk, hk = pair % a.hk;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   const int col0 = wave * kDW;
 
@@ -619,8 +627,13 @@ __global__ __launch_bounds__(kFNT) void bwd_dq_d512_kernel(const BwdArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb = wave / kNW, cw = wave % kNW;             // row block, column share
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, h = blockIdx.y;
-  const int mt = gridDim.x - 1 - blockIdx.x;              // most visible keys first (causal)
+  // one workgroup per (sequence, q-head, Q tile): the tiles of a kv-head's group back to back on one
+  // XCD, most visible keys (causal) first
+  const int nmt = (a.seq.max_seqlen_q + kFBR - 1) / kFBR, group = a.hq / a.hk;
+  int pair, r_item;
+  if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, group * nmt, pair, r_item)) return;
+  const int z = pair / a.hk, h = (pair % a.hk) * group + r_item % group;
+  const int mt = nmt - 1 - r_item / group;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   const int col0 = cw * kDW;
   float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * 2 * (Smem512::PART_BYTES / 4);
@@ -801,10 +814,6 @@ __global__ __launch_bounds__(kFNT) void bwd_dq_d512_kernel(const BwdArgs a) {
   }
 }
 
-int nseq_of(const SeqArgs& s, int batch) {
-  return s.num_seqlens != 0 ? (s.num_seqlens < 0 ? -s.num_seqlens : s.num_seqlens) : batch;
-}
-
 template <auto kern, int NT = kNT, typename Args>
 hipError_t launch512(dim3 grid, int smem, hipStream_t stream, const Args& a) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;   // an empty tensor: nothing to write
@@ -829,7 +838,7 @@ hipError_t launch512(dim3 grid, int smem, hipStream_t stream, const Args& a) {
 
 template <typename T>
 hipError_t run_fwd_t(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
-  const dim3 grid((a.seq.max_seqlen_q + kFBR - 1) / kFBR, a.hq, nseq_of(a.seq, a.batch));
+  const dim3 grid(xcd_grid(nseq_of(a.seq, a.batch) * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + kFBR - 1) / kFBR)));
   constexpr int smem = SmemFwd512::BYTES;
 #define FA_CALL(W, B, P) launch512<fwd_d512_kernel<T, W, B, P>, kFNT>(grid, smem, s, a)
   FA_D512_SWITCH(FA_CALL)
@@ -840,13 +849,13 @@ template <typename T>
 hipError_t run_bwd_t(int kernel_slot, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
   const int nseq = nseq_of(a.seq, a.batch);
   if (kernel_slot == 1) {
-    const dim3 grid((a.seq.max_seqlen_k + kBR - 1) / kBR, a.hk, nseq);
+    const dim3 grid(xcd_grid(nseq * a.hk, (a.seq.max_seqlen_k + kBR - 1) / kBR));
 #define FA_CALL(W, B, P) launch512<bwd_dkdv_d512_kernel<T, W, B, P>>(grid, SmemBwd512::BYTES, s, a)
     FA_D512_SWITCH(FA_CALL)
 #undef FA_CALL
   }
   if (kernel_slot == 2) {
-    const dim3 grid((a.seq.max_seqlen_q + kFBR - 1) / kFBR, a.hq, nseq);
+    const dim3 grid(xcd_grid(nseq * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + kFBR - 1) / kFBR)));
 #define FA_CALL(W, B, P) launch512<bwd_dq_d512_kernel<T, W, B, P>, kFNT>(grid, SmemDq512::BYTES, s, a)
     FA_D512_SWITCH(FA_CALL)
 #undef FA_CALL

@@ -287,6 +287,24 @@ __device__ __forceinline__ void split_zh(int zh, int nseq, int group, int& z, in
   h = (t / nseq) * group + g;
 }
 
+// 1-D grids of the kernels that launch one workgroup per tile.  Consecutive workgroup ids go round
+// the 8 XCDs, so XCD x = id % 8 takes the (sequence, kv-head) pairs x, x + 8, ... one after the
+// other and the `per` tiles of a pair back to back: what every tile of a pair streams (its K/V, or
+// the Q/dO of the group's q-heads) then stays in that XCD's L2.  Handed out tile by tile in grid
+// order, the workgroups of one pair landed on all XCDs and drifted apart under a causal mask, and
+// each streamed from HBM on its own (head dim 512, S = 4096: causal forward 3.39 ms against 2.31 for
+// half of the non-causal one).  Returns false past the last pair.
+__device__ __forceinline__ bool xcd_item(int id, int pairs, int per, int& pair, int& r) {
+  const int xcd = id % kNumXcd, idx = id / kNumXcd;
+  pair = xcd + kNumXcd * (idx / per);
+  r = idx % per;
+  return pair < pairs;
+}
+inline int xcd_grid(int pairs, int per) { return kNumXcd * ((pairs + kNumXcd - 1) / kNumXcd) * per; }
+__host__ __device__ inline int nseq_of(const SeqArgs& s, int batch) {
+  return s.num_seqlens != 0 ? (s.num_seqlens < 0 ? -s.num_seqlens : s.num_seqlens) : batch;
+}
+
 // _lse_offset, modules/flash/kernel/fwd_kernel_inner.py:38-43
 __device__ __forceinline__ int64_t lse_offset(const SeqInfo& si, int h, int hq) {
   return ((int64_t)si.batch_index * hq + h) * si.lse_stride + si.q_start;

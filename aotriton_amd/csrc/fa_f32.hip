@@ -147,17 +147,15 @@ __device__ __forceinline__ void col_gemm(const float* tile, int c, int hi, int c
   }
 }
 
-struct WindowOf {
-  Window w;
-  template <bool kWindowed>
-  __device__ __forceinline__ static Window get(const MaskArgs& m, int sq, int sk) {
-    Window w{0, 0};
-    if (kWindowed) w = parse_window(m.causal_type, m.window_left, m.window_right, sq, sk);
-    w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
-    w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
-    return w;
-  }
-};
+// the window of a sequence, kept inside int32 when added to a row or a key
+template <bool kWindowed>
+__device__ __forceinline__ Window window_of(const MaskArgs& m, int sq, int sk) {
+  Window w{0, 0};
+  if (kWindowed) w = parse_window(m.causal_type, m.window_left, m.window_right, sq, sk);
+  w.left = w.left > (1 << 30) ? (1 << 30) : (w.left < -(1 << 30) ? -(1 << 30) : w.left);
+  w.right = w.right > (1 << 30) ? (1 << 30) : (w.right < -(1 << 30) ? -(1 << 30) : w.right);
+  return w;
+}
 
 // ---------------------------------------------------------------------------------------------
 // forward: one workgroup = 64 query rows of one head = 8 waves, four per 32-row block
@@ -181,11 +179,16 @@ __global__ __launch_bounds__(kNT2) void fwd_f32_kernel(const FwdArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb = wave / kNW, cw = wave % kNW;             // row block, column share
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, h = blockIdx.y;
-  const int mt = gridDim.x - 1 - blockIdx.x;              // most visible keys first (causal)
+  // one workgroup per (sequence, q-head, Q tile): the tiles of a kv-head's group back to back on one
+  // XCD, most visible keys (causal) first
+  const int nmt = (a.seq.max_seqlen_q + kBR2 - 1) / kBR2, group = a.hq / a.hk;
+  int pair, r_item;
+  if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, group * nmt, pair, r_item)) return;
+  const int z = pair / a.hk, h = (pair % a.hk) * group + r_item % group;
+  const int mt = nmt - 1 - r_item / group;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   float* part = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * (kPartBytes / 4);
-  if (kDropout && blockIdx.x == 0 && h == 0 && z == 0 && tid == 0) {
+  if (kDropout && blockIdx.x == 0 && tid == 0) {
     // modules/flash/kernel/fwd_kernel.py:199-207
     uint64_t base = a.drop.offset2;
     if (a.drop.offset1_ptr) base += *a.drop.offset1_ptr;
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(kNT2) void fwd_f32_kernel(const FwdArgs a) {
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * kBR2;
   if (q0 >= si.seqlen_q) return;
-  const Window w = WindowOf::get<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
+  const Window w = window_of<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
   const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kBR2, kBC);
 
   const int hk = h / (a.hq / a.hk);                       // fwd_kernel.py:360
@@ -393,14 +396,18 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_f32_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, hk = blockIdx.y, nt = blockIdx.x;
+  // one workgroup per (sequence, kv-head, key block): the key blocks of a kv-head back to back on
+  // one XCD, those that the most queries see (causal) first
+  int pair, nt;
+  if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, (a.seq.max_seqlen_k + kBC - 1) / kBC, pair, nt)) return;
+  const int z = pair / a.hk, hk = pair % a.hk;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   const int col0 = wave * C::DW;
 
   const SeqInfo si = get_seq(a.seq, z);
   const int n0 = nt * kBC;
   if (n0 >= si.seqlen_k) return;
-  const Window w = WindowOf::get<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
+  const Window w = window_of<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
   // rows are keys here, columns are queries: key n sees query m iff n - right <= m <= n + left
   // (bwd_kernel_dk_dv.py:268-279 passes the window transposed in the same way)
   const BlockRanges br = block_ranges(kWindowed, w.right, w.left, n0, si.seqlen_k, si.seqlen_q, kBC, kBC);
@@ -572,8 +579,13 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb = wave / kNW, cw = wave % kNW;             // row block, column share
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
-  const int z = blockIdx.z, h = blockIdx.y;
-  const int mt = gridDim.x - 1 - blockIdx.x;              // most visible keys first (causal)
+  // one workgroup per (sequence, q-head, Q tile): the tiles of a kv-head's group back to back on one
+  // XCD, most visible keys (causal) first
+  const int nmt = (a.seq.max_seqlen_q + kBR2 - 1) / kBR2, group = a.hq / a.hk;
+  int pair, r_item;
+  if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, group * nmt, pair, r_item)) return;
+  const int z = pair / a.hk, h = (pair % a.hk) * group + r_item % group;
+  const int mt = nmt - 1 - r_item / group;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   const int col0 = cw * C::DW;
   float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * 2 * (kPartBytes / 4);
@@ -583,7 +595,7 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
   const SeqInfo si = get_seq(a.seq, z);
   const int q0 = mt * kBR2;
   if (q0 >= si.seqlen_q) return;
-  const Window w = WindowOf::get<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
+  const Window w = window_of<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
   const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kBR2, kBC);
 
   const int hk = h / (a.hq / a.hk);
@@ -728,10 +740,6 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
   }
 }
 
-int nseq_of(const SeqArgs& s, int batch) {
-  return s.num_seqlens != 0 ? (s.num_seqlens < 0 ? -s.num_seqlens : s.num_seqlens) : batch;
-}
-
 template <auto kern, int NT, typename Args>
 hipError_t launch(dim3 grid, int smem, hipStream_t stream, const Args& a) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;   // an empty tensor: nothing to write
@@ -758,7 +766,7 @@ hipError_t launch(dim3 grid, int smem, hipStream_t stream, const Args& a) {
 
 template <int D>
 hipError_t run_fwd_d(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
-  const dim3 grid((a.seq.max_seqlen_q + kBR2 - 1) / kBR2, a.hq, nseq_of(a.seq, a.batch));
+  const dim3 grid(xcd_grid(nseq_of(a.seq, a.batch) * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + kBR2 - 1) / kBR2)));
 #define FA_CALL(W, B, P) launch<fwd_f32_kernel<D, W, B, P>, kNT2>(grid, SmemFwd<D>::BYTES, s, a)
   FA_F32_SWITCH(FA_CALL)
 #undef FA_CALL
@@ -768,13 +776,13 @@ template <int D>
 hipError_t run_bwd_d(int kernel_slot, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
   const int nseq = nseq_of(a.seq, a.batch);
   if (kernel_slot == 1) {
-    const dim3 grid((a.seq.max_seqlen_k + kBC - 1) / kBC, a.hk, nseq);
+    const dim3 grid(xcd_grid(nseq * a.hk, (a.seq.max_seqlen_k + kBC - 1) / kBC));
 #define FA_CALL(W, B, P) launch<bwd_dkdv_f32_kernel<D, W, B, P>, kNT>(grid, SmemDkDv<D>::BYTES, s, a)
     FA_F32_SWITCH(FA_CALL)
 #undef FA_CALL
   }
   if (kernel_slot == 2) {
-    const dim3 grid((a.seq.max_seqlen_q + kBR2 - 1) / kBR2, a.hq, nseq);
+    const dim3 grid(xcd_grid(nseq * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + kBR2 - 1) / kBR2)));
 #define FA_CALL(W, B, P) launch<bwd_dq_f32_kernel<D, W, B, P>, kNT2>(grid, SmemDq<D>::BYTES, s, a)
     FA_F32_SWITCH(FA_CALL)
 #undef FA_CALL

@@ -310,10 +310,6 @@ __global__ void valu_dkdv_kernel(const BwdArgs a) {
   store_row<DPL, T>(dvp, dv, sub, a.head_dim_v, 1.0f);
 }
 
-int nseq_of(const SeqArgs& s, int batch) {
-  return s.num_seqlens != 0 ? (s.num_seqlens < 0 ? -s.num_seqlens : s.num_seqlens) : batch;
-}
-
 }  // namespace
 
 // head_dim: 64, 128, 256 or 512, the one that holds the tensors' head dims.  The 16-bit types

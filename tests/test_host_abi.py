@@ -115,7 +115,7 @@ def test_validate_fwd_error_contract():
     assert validate_fwd(p6, 3) == E.hipErrorInvalidValue
     p7, k7 = _fwd_params(D=512)                                                # above 256: the head dim split over the waves, 64 rows per workgroup
     err, cfg = query_fwd_config(p7)
-    assert err == E.hipSuccess and cfg.head_dim == 512 and cfg.block_m == 64 and list(cfg.grid) == [1, 4, 2]
+    assert err == E.hipSuccess and cfg.head_dim == 512 and cfg.block_m == 64 and list(cfg.grid) == [16, 1, 1]
     for bad in (520, 100):                                                     # > 512, or rows not a multiple of 16 bytes
         pb, kb = _fwd_params(D=bad)
         assert validate_fwd(pb, 3) == E.hipErrorNotSupported
