@@ -287,6 +287,47 @@ __device__ __forceinline__ void split_zh(int zh, int nseq, int group, int& z, in
   h = (t / nseq) * group + g;
 }
 
+// The list of work items of one XCD when the sequences differ in length.  The dense list of the
+// persistent kernels has a slot for every tile up to the longest sequence, most of them empty for
+// the short ones, and which worker draws the empty slots is systematic (16 packed sequences of
+// 256-8192 tokens: the busiest forward worker had 19 % more K tiles than the average).  This list
+// holds the valid tiles only: the heads zh of the XCD set by set (a set = the `ratio` heads that
+// share K/V, or Q/dO: the q-heads of one kv-head of one sequence), a set's tiles one after the
+// other with its heads interleaved.  A worker asks for positions t in increasing order.
+struct RaggedWalk {
+  int lo, hi, ratio, nseq, rows_per_tile;
+  bool keys;                       // tiles count keys (dK/dV) instead of queries
+  int set, set_end, base, first, members, tiles;
+  __device__ __forceinline__ void open(const SeqArgs& seq) {
+    first = lo > set * ratio ? lo : set * ratio;
+    members = (hi < (set + 1) * ratio ? hi : (set + 1) * ratio) - first;
+    const SeqInfo si = get_seq(seq, set % nseq);
+    tiles = ((keys ? si.seqlen_k : si.seqlen_q) + rows_per_tile - 1) / rows_per_tile;
+  }
+  __device__ __forceinline__ void init(const SeqArgs& seq, int xcd, int zh_per_xcd, int num_zh, int ratio_, int nseq_,
+                                       int rows_per_tile_, bool keys_) {
+    lo = xcd * zh_per_xcd;
+    hi = lo + zh_per_xcd < num_zh ? lo + zh_per_xcd : num_zh;
+    ratio = ratio_; nseq = nseq_; rows_per_tile = rows_per_tile_; keys = keys_;
+    set = lo / ratio; set_end = (hi + ratio - 1) / ratio;
+    base = 0; first = 0; members = 0; tiles = 0;
+    if (set < set_end) open(seq);
+  }
+  // head zh and tile index (counted from the sequence's start) at position t; false past the end
+  __device__ __forceinline__ bool at(const SeqArgs& seq, int t, int& zh, int& tile) {
+    while (set < set_end && t >= base + members * tiles) {
+      base += members * tiles;
+      if (++set < set_end) open(seq);
+    }
+    if (set >= set_end) return false;
+    const int off = t - base;
+    zh = first + off % members;
+    tile = off / members;
+    return true;
+  }
+  __device__ __forceinline__ int tiles_of_set() const { return tiles; }
+};
+
 // 1-D grids of the kernels that launch one workgroup per tile.  Consecutive workgroup ids go round
 // the 8 XCDs, so XCD x = id % 8 takes the (sequence, kv-head) pairs x, x + 8, ... one after the
 // other and the `per` tiles of a pair back to back: what every tile of a pair streams (its K/V, or

@@ -578,43 +578,26 @@ void fwd_kernel(const FwdArgs a) {
   const int workers = gridDim.x / kNumXcd;
   const int per_group = a.zh_group * a.num_m_tiles;
   const int items = a.items_per_xcd;
-  // Sequences of different lengths: the dense list has num_m_tiles slots per head, most of them
-  // empty for the short sequences, and which worker draws the empty ones is systematic (16 packed
-  // sequences of 256-8192 tokens: the busiest worker had 19 % more K tiles than the average).  The
-  // list then holds the valid tiles only: the heads of this XCD set by set (a set = the q-heads of
-  // one kv-head of one sequence, which share K/V), a set's tiles from the last one down with its
-  // heads interleaved; the workers take it in the same serpentine order.
+  // sequences of different lengths: the list of the valid tiles only (RaggedWalk), a set's tiles
+  // from the last one down; taken in the same serpentine order
   const bool ragged = a.seq.num_seqlens != 0;
   const int ratio = a.hq / a.hk, nseq = a.num_zh / a.hq;
-  const int zh_lo = xcd * a.zh_per_xcd;
-  const int zh_hi = zh_lo + a.zh_per_xcd < a.num_zh ? zh_lo + a.zh_per_xcd : a.num_zh;
-  constexpr int BM_ = NW * 32 * (QB > 0 ? QB : 1);
-  int set = zh_lo / ratio, base = 0, first = 0, members = 0, tiles = 0;
-  const int set_end = (zh_hi + ratio - 1) / ratio;
-  auto open_set = [&]() {
-    first = zh_lo > set * ratio ? zh_lo : set * ratio;
-    members = (zh_hi < (set + 1) * ratio ? zh_hi : (set + 1) * ratio) - first;
-    tiles = (get_seq(a.seq, set % nseq).seqlen_q + BM_ - 1) / BM_;
-  };
-  if (ragged && set < set_end) open_set();
+  RaggedWalk walk;
+  if (ragged) walk.init(a.seq, xcd, a.zh_per_xcd, a.num_zh, ratio, nseq, NW * 32 * (QB > 0 ? QB : 1), false);
   for (int r = 0;; ++r) {
     const int t = r * workers + ((r & 1) ? workers - 1 - p : p);
     int z, h, mt;
     if (ragged) {
-      while (set < set_end && t >= base + members * tiles) {
-        base += members * tiles;
-        if (++set < set_end) open_set();
-      }
-      if (set >= set_end) break;
-      const int off = t - base;
-      split_zh(first + off % members, nseq, ratio, z, h);
-      mt = tiles - 1 - off / members;
+      int zh, tile;
+      if (!walk.at(a.seq, t, zh, tile)) break;
+      split_zh(zh, nseq, ratio, z, h);
+      mt = walk.tiles_of_set() - 1 - tile;
     } else {
       if (r * workers >= items) break;
       if (t >= items) continue;
       const int gi = t / per_group, gr = t % per_group;
       const int zh_local = gi * a.zh_group + gr % a.zh_group;
-      const int zh = zh_lo + zh_local;
+      const int zh = xcd * a.zh_per_xcd + zh_local;
       if (zh_local >= a.zh_per_xcd || zh >= a.num_zh) continue;
       mt = a.num_m_tiles - 1 - gr / a.zh_group;
       split_zh(zh, nseq, ratio, z, h);
