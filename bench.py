@@ -393,6 +393,33 @@ def main():
         del q5, k5, v5, do5, b5, db5
         torch.cuda.empty_cache()
 
+        # --- the two other kernel families: head dim 512 (bf16) and fp32 tensors, causal ---------------
+        def family(Bx, Hx, Sx, Dx, dt, peak):
+            rnx = lambda: torch.randn(Bx, Hx, Sx, Dx, device=dev, dtype=torch.float32, generator=gg).to(dt)
+            qx, kx, vx, dox = rnx(), rnx(), rnx(), rnx()
+            ox, dqx, dkx, dvx = (torch.empty_like(qx) for _ in range(4))
+            Lx = torch.empty(Bx * Hx, Sx, device=dev, dtype=torch.float32)
+            dx = torch.empty_like(Lx)
+            smx = 1.0 / math.sqrt(Dx)
+
+            def fwdx():
+                assert flash.attn_fwd(qx, kx, vx, None, smx, Lx, ox, 0.0, null, null, 0, null, null, None, True, atomic) == ok
+
+            def bwdx():
+                assert flash.attn_bwd(qx, kx, vx, None, smx, ox, dox, dqx, dkx, dvx, None, None, Lx, dx, 0.0, null, null,
+                                      0, True) == ok
+
+            flx = 4.0 * Bx * Hx * Sx * Sx * Dx * 0.5
+            rf, rb = do_bench(fwdx, max_reps=30), do_bench(bwdx, max_reps=12)
+            return {'fwd': {'ms': rf['median'], 'tflops': tf(flx, rf['median']), 'frac_peak': tf(flx, rf['median']) / peak},
+                    'bwd_split': {'ms': rb['median'], 'tflops': tf(2.5 * flx, rb['median']),
+                                  'frac_peak': tf(2.5 * flx, rb['median']) / peak},
+                    'peak_tflops_used': peak}
+
+        out['d512'] = {'workload': 'B=4 H=16 S=4096 D=512 bf16 causal', **family(4, 16, 4096, 512, torch.bfloat16, PEAK_BF16_TFLOPS)}
+        out['fp32'] = {'workload': 'B=4 H=32 S=4096 D=128 fp32 causal (fp32 MFMA peak)',
+                       **family(4, 32, 4096, 128, torch.float32, 157.3)}
+
     if not args.no_cpu:
         out['cpu_baseline'] = cpu_baseline(B, H, S, D, causal, seed)
     print(json.dumps(out))
