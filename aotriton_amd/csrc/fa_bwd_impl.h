@@ -1311,17 +1311,34 @@ void bwd_dkdv_kernel(const BwdArgs a) {
   // 2P-1-p, 2P+p, ...), which pairs heavy with light items.
   const int xcd = blockIdx.x % kNumXcd, p = blockIdx.x / kNumXcd, workers = gridDim.x / kNumXcd;
   const int per_group = a.zh_group * a.num_n_tiles;
+  // Sequences of different lengths: the valid tiles only, heaviest first (LevelWalk), taken in the
+  // same serpentine order.
+  const bool ragged = dkdv_level_list<D>(a);
+  const int zh_lo = xcd * a.zh_per_xcd;
+  LevelWalk walk;
+  if (ragged)
+    walk.init<NW * 64>(reinterpret_cast<uint32_t*>(smem_raw + DkDvSmem<D, BM>::BYTES), a.seq, zh_lo,
+                       zh_lo + a.zh_per_xcd < a.num_zh ? zh_lo + a.zh_per_xcd : a.num_zh, a.num_zh / a.hk, NW * 32, true,
+                       threadIdx.x);
   // (D = 256 is launched with one workgroup per item: the loop would cost registers there)
   for (int r = 0; D >= 256 ? r < 1 : r * workers < a.items_per_xcd; ++r) {
     const int li = r * workers + ((r & 1) ? workers - 1 - p : p);
-    if (li >= a.items_per_xcd) continue;
-    const int gi = li / per_group, gr = li % per_group;
-    const int zl = gi * a.zh_group + gr % a.zh_group;
-    const int zh = xcd * a.zh_per_xcd + zl;
-    if (zl >= a.zh_per_xcd || zh >= a.num_zh) continue;
+    int zh, nt;
+    if (ragged) {
+      int e;
+      if (!walk.at(li, e, nt)) break;
+      zh = zh_lo + e;
+    } else {
+      if (li >= a.items_per_xcd) continue;
+      const int gi = li / per_group, gr = li % per_group;
+      const int zl = gi * a.zh_group + gr % a.zh_group;
+      zh = zh_lo + zl;
+      if (zl >= a.zh_per_xcd || zh >= a.num_zh) continue;
+      nt = gr / a.zh_group;
+    }
     int z, hk;
     split_zh(zh, a.num_zh / a.hk, 1, z, hk);
-    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad>(a, hk, gr / a.zh_group, z, smem_raw);
+    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad>(a, hk, nt, z, smem_raw);
     __syncthreads();     // the next item reuses the LDS stages
   }
 }
@@ -1400,6 +1417,13 @@ inline int bwd_nseq(const BwdArgs& a) {
 // grid was 10 % slower, while it gains 1 % at the headline shape and 12 % on packed
 // sequences of very different lengths.  D = 256 also gets one workgroup per item: its
 // dK/dV kernel has no register to spare for the loop.
+// Whether the dK/dV kernel walks the level list: persistent workgroups over sequences of different
+// lengths, few enough (sequence, kv-head) entries per XCD for the table.
+template <int D>
+__host__ __device__ inline bool dkdv_level_list(const BwdArgs& a) {
+  return D < 256 && a.seq.num_seqlens != 0 && a.bias == nullptr && a.zh_per_xcd <= kLevelCap && a.num_n_tiles <= 0xffff;
+}
+
 template <int D>
 inline int persistent_workers(const BwdArgs& a) {
   if (a.bias != nullptr || D >= 256) return a.items_per_xcd;
@@ -1452,7 +1476,9 @@ hipError_t launch_dkdv_variant(const BwdArgs& a0, hipStream_t stream) {
   a.zh_group = 2;
   a.items_per_xcd = ((a.zh_per_xcd + a.zh_group - 1) / a.zh_group) * a.zh_group * a.num_n_tiles;
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
-  return launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>>(grid, NW * 64, DkDvSmem<D, BM>::BYTES, stream, a);
+  // (the level table's LDS is requested whether or not this launch uses it: the kernel's limit is set once)
+  constexpr int smem = DkDvSmem<D, BM>::BYTES + (D < 256 ? kLevelBytes : 0);
+  return launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>>(grid, NW * 64, smem, stream, a);
 }
 
 template <typename T, int D, bool kPad>
@@ -1513,7 +1539,7 @@ template <typename T, int D, bool kWindowed> TileShape bwd_shape(int slot) {
   constexpr int s1 = DkDvSmem<D, BM>::BYTES, s2 = DqSmem<D, BN>::BYTES;
   switch (slot) {
     case 0: return TileShape{256 / (D / 8), 0, 4, 0};
-    case 1: return TileShape{BM, NW * 32, NW, s1};
+    case 1: return TileShape{BM, NW * 32, NW, s1 + (D < 256 ? kLevelBytes : 0)};
     case 2: return TileShape{NW * 32, BN, NW, s2};
     default: return TileShape{NW * 32, NW * 32, NW, s1 > s2 ? s1 : s2};
   }
