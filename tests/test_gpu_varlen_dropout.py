@@ -119,6 +119,21 @@ def test_compact_varlen_with_empty_sequences(dtype, causal, backend):
     _run_varlen_case([5, 0, 70, 0, 33, 130], [9, 64, 0, 0, 33, 40], 4, 2, 64, dtype, causal, backend)
 
 
+@pytest.mark.parametrize('nseq,hk', [(67, 1), (300, 2), (4200, 1)])
+@pytest.mark.parametrize('causal', [True, (40, 0)])
+def test_many_packed_sequences(nseq, hk, causal):
+    # The dK/dV kernel sorts the (sequence, kv-head) entries of an XCD by length into an LDS table of
+    # 512 entries and walks the valid key tiles heaviest first; beyond 512 entries per XCD it keeps the
+    # dense list.  9, 75 and 525 entries per XCD, lengths from empty to several key tiles, equal
+    # lengths among them.
+    rng = np.random.default_rng(nseq)
+    hi = 700 if nseq < 100 else (300 if nseq < 1000 else 40)
+    lens = rng.integers(0, hi, size=nseq)
+    lens[::7] = 129
+    lens[3] = 0
+    _run_varlen_case(lens, lens, 2 * hk, hk, 64, torch.bfloat16, causal, 0)
+
+
 def _sampled_varlen_cases(n=40, seed=4242):
     """Seeded packed-sequence cases: 1-6 sequences of 0-300 tokens (the reference draws its
     lengths from a fixed list, tests/test_varlen.py:34-47), key lengths that differ from the
