@@ -41,9 +41,16 @@ struct Cfg {
   static constexpr int DW = D / kNW;      // columns a wave owns
   static constexpr int KJ = DW / 8;       // 16-byte pieces of a lane per row (each feeds four MFMAs)
   static constexpr int DB = DW / 32;      // 32-column blocks a wave owns
-  static constexpr int STR = D + 8;       // floats per tile row in LDS
+  static constexpr int STR = D;           // floats per tile row in LDS (unpadded, pieces swizzled)
   static constexpr int TILE_BYTES = kBC * STR * 4;
 };
+
+// LDS tiles keep the 16-byte piece q of row r at piece position q ^ swz(r).  Two access patterns must
+// sweep the 64 banks once: a quarter-wave reading one piece each of 16 consecutive rows (swz is a
+// bijection on r % 16), and a wave reading 32 consecutive floats each of two rows four apart (bit 3 of
+// swz is bit 2 of r, so the two rows' eight pieces fall into different halves of the banks).  With
+// padded rows instead, one of the two patterns always pairs up lanes on a bank.
+__device__ __forceinline__ int swz(int r) { return (r & 3) | (((r >> 2) & 1) << 3) | (((r >> 3) & 1) << 2); }
 
 __device__ __forceinline__ f32x16 mfma32(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -110,7 +117,8 @@ struct TileFetch {
   __device__ __forceinline__ void store(float* lds, int tid) const {
     const int r0 = tid / LPR, cc0 = tid % LPR;
 #pragma unroll
-    for (int i = 0; i < CH; ++i) *reinterpret_cast<f32x4*>(lds + (r0 + i * RPI) * Cfg<D>::STR + cc0 * 4) = reg[i];
+    for (int i = 0; i < CH; ++i)
+      *reinterpret_cast<f32x4*>(lds + (r0 + i * RPI) * Cfg<D>::STR + (cc0 ^ swz(r0 + i * RPI)) * 4) = reg[i];
   }
 };
 
@@ -126,10 +134,11 @@ __device__ __forceinline__ void load_resident(f32x4 (&reg)[Cfg<D>::KJ], const fl
 template <int D>
 __device__ __forceinline__ f32x16 row_gemm(const float* tile, int c, int hi, int col0,
                                            const f32x4 (&res)[Cfg<D>::KJ], f32x16 acc) {
-  const float* p = tile + c * Cfg<D>::STR + col0 + 4 * hi;
+  const float* p = tile + c * Cfg<D>::STR;
+  const int q0 = col0 / 4 + hi, sw = swz(c);
 #pragma unroll
   for (int j = 0; j < Cfg<D>::KJ; ++j) {
-    const f32x4 a4 = *reinterpret_cast<const f32x4*>(p + 8 * j);
+    const f32x4 a4 = *reinterpret_cast<const f32x4*>(p + ((q0 + 2 * j) ^ sw) * 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc = mfma32(a4[e], res[j][e], acc);
   }
@@ -141,9 +150,11 @@ __device__ __forceinline__ void col_gemm(const float* tile, int c, int hi, int c
                                          f32x16 (&acc)[Cfg<D>::DB]) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    const float* p = tile + (8 * (i / 4) + 4 * hi + (i % 4)) * Cfg<D>::STR + col0 + c;
+    const int r = 8 * (i / 4) + 4 * hi + (i % 4);
+    const float* p = tile + r * Cfg<D>::STR + (c & 3);
+    const int q0 = (col0 + c) / 4, sw = swz(r);
 #pragma unroll
-    for (int db = 0; db < Cfg<D>::DB; ++db) acc[db] = mfma32(p[32 * db], x[i], acc[db]);
+    for (int db = 0; db < Cfg<D>::DB; ++db) acc[db] = mfma32(p[((q0 + 8 * db) ^ sw) * 4], x[i], acc[db]);
   }
 }
 
