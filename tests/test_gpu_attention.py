@@ -338,6 +338,40 @@ def test_sampled_strides_bias_layouts_and_masks(i):
         check('db', bg.grad, rg[3], lg[3], FUDGE['db'])
 
 
+@pytest.mark.parametrize('dtype,D', [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 256), (torch.bfloat16, 512),
+                                     (torch.float32, 128), (torch.float32, 320), (torch.bfloat16, 72)])
+@pytest.mark.parametrize('causal', [False, True])
+def test_delta_is_the_row_sum_of_o_times_do(dtype, D, causal):
+    """bwd_preprocess (modules/flash/kernel/bwd_preprocess.py:28-133): delta[z, h, m] = sum_d fp32(O) fp32(dO),
+    laid out like the LSE.  The split backward leaves it in the caller's buffer whichever kernel computes it
+    (the dQ kernel at head dims up to 256, the preprocess kernel otherwise), and the preprocess kernel
+    launched on its own writes the same.  Closed form, computed here in fp64."""
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton.v3.flash import attn_bwd_kernel, attn_bwd_params
+    B, Hq, Hk, Sq, Sk = 2, 4, 2, 203, 261
+    q, k, v, _, do = make_inputs(B, Hq, Hk, Sq, Sk, D, dtype, DEV, seed=5)
+    sm = 1.0 / math.sqrt(D)
+    ok = flash.hipError_t.hipSuccess
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    o = torch.empty_like(q)
+    L = torch.empty(B * Hq, Sq, device=DEV, dtype=torch.float32)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+    assert flash.attn_fwd(q, k, v, None, sm, L, o, 0.0, null, null, 0, null, null, None, causal, atomic) == ok
+    want = (o.double() * do.double()).sum(-1).view(B * Hq, Sq)
+    tol = 1e-5 * max(1.0, want.abs().max().item())
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    delta = torch.full_like(L, float('nan'))
+    assert flash.attn_bwd(q, k, v, None, sm, o, do, dq, dk, dv, None, None, L, delta, 0.0, null, null, 0, causal) == ok
+    torch.cuda.synchronize()
+    assert (delta.double() - want).abs().max().item() <= tol
+    alone = torch.full_like(L, float('nan'))
+    bp = attn_bwd_params()
+    flash._fill_bwd(bp, q, k, v, None, sm, o, do, dq, dk, dv, None, None, L, alone, 0.0, null, null, 0, causal)
+    assert attn_bwd_kernel(bp, attn_bwd_params.kVersion, flash._stream(), 0) == ok
+    torch.cuda.synchronize()
+    assert (alone.double() - want).abs().max().item() <= tol
+
+
 def test_concurrent_streams_and_threads_give_the_serial_results():
     """Calls are re-entrant and ordered only by the stream they are given: three host threads,
     each on its own stream with its own shape, repeat forward + backward; every result must
