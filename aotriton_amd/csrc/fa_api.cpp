@@ -107,16 +107,21 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 constexpr int64_t kMaxRowStride = 1 << 21;   // elements; 256 rows of it stay below 2^31 bytes at 4 bytes per element
 
-// rank-4 activation tensor: non-null unless it has no element, unit last stride, 16-byte aligned rows
-int check_act(const fa_tensor4& t, int dtype) {
+// rank-4 activation tensor: non-null unless it has no element, unit last stride.  *pieces is cleared
+// when its rows are not made of aligned 16-byte pieces (a head dim or a stride that is no multiple
+// of 8 elements, a base address that is not 16-byte aligned): such tensors run on the kernels that
+// move single elements (the reference masks the excess columns of any head dim, attn_fwd.cc:76-82).
+int check_act(const fa_tensor4& t, int dtype, bool* pieces) {
   const bool empty = (t.sizes[0] == 0 || t.sizes[1] == 0 || t.sizes[2] == 0) && t.sizes[3] > 0;
   if (t.ptr == nullptr && !empty) return FA_ERROR_INVALID_VALUE;
   if (t.dtype != dtype) return FA_ERROR_INVALID_VALUE;
   if (t.strides[3] != 1) return FA_ERROR_NOT_SUPPORTED;
-  if (!aligned16(t.ptr)) return FA_ERROR_NOT_SUPPORTED;
+  if (!aligned16(t.ptr) || t.sizes[3] % 8 != 0) *pieces = false;
   // strides travel as unsigned 64-bit numbers; one above 2^63 is a negative stride
-  for (int i = 0; i < 3; ++i)
-    if (t.sizes[i] > 1 && ((t.strides[i] % 8) != 0 || (int64_t)t.strides[i] < 0)) return FA_ERROR_NOT_SUPPORTED;
+  for (int i = 0; i < 3; ++i) {
+    if (t.sizes[i] > 1 && (int64_t)t.strides[i] < 0) return FA_ERROR_NOT_SUPPORTED;
+    if (t.sizes[i] > 1 && (t.strides[i] % 8) != 0) *pieces = false;
+  }
   // a tile's rows are addressed with 32-bit byte offsets from the tile's first row
   if (t.sizes[2] > 1 && (int64_t)t.strides[2] > kMaxRowStride) return FA_ERROR_NOT_SUPPORTED;
   return FA_SUCCESS;
@@ -140,6 +145,7 @@ fa::Strides3 strides3(const fa_tensor4& t) {
 struct Shape {
   int batch, hq, hk, d, d_qk, d_v, max_sq, max_sk, num_seqlens;  // d: compiled head dim; d_qk, d_v: the tensors'; num_seqlens signed as in attn_fwd.cc:99
   bool windowed, bias, dropout;
+  bool elementwise;       // some activation tensor is not made of aligned 16-byte pieces
   int64_t row_stats;      // elements of L and of delta
 };
 
@@ -153,10 +159,12 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   if (dtype != FA_DTYPE_FLOAT16 && dtype != FA_DTYPE_BFLOAT16 && dtype != FA_DTYPE_FLOAT32)
     return FA_ERROR_INVALID_VALUE;
   int e;
-  if ((e = check_act(Q, dtype)) != FA_SUCCESS) return e;
-  if ((e = check_act(K, dtype)) != FA_SUCCESS) return e;
-  if ((e = check_act(V, dtype)) != FA_SUCCESS) return e;
+  bool pieces = true;
+  if ((e = check_act(Q, dtype, &pieces)) != FA_SUCCESS) return e;
+  if ((e = check_act(K, dtype, &pieces)) != FA_SUCCESS) return e;
+  if ((e = check_act(V, dtype, &pieces)) != FA_SUCCESS) return e;
   Shape s{};
+  s.elementwise = !pieces;
   s.batch = (int)Q.sizes[0];
   s.hq = (int)Q.sizes[1];
   s.hk = (int)K.sizes[1];
@@ -168,7 +176,7 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   // Head dims are rounded up to a compiled one and the excess columns are masked in
   // the kernels (PADDED_HEAD, attn_fwd.cc:76-82,109); 16-byte granularity.  Dqk and Dv
   // may differ: both run on the compiled head dim that holds the larger one.
-  if (dqk <= 0 || dqk > 512 || dqk % 8 != 0 || dv <= 0 || dv > 512 || dv % 8 != 0) return FA_ERROR_NOT_SUPPORTED;
+  if (dqk <= 0 || dqk > 512 || dv <= 0 || dv > 512) return FA_ERROR_NOT_SUPPORTED;
   s.d_qk = dqk;
   s.d_v = dv;
   const int dmax = dqk > dv ? dqk : dv;
@@ -240,7 +248,9 @@ int validate_fwd(const fa_fwd_params* p, int32_t version, const fa_options* opt,
                        p->seq_strides_k, p->Max_seqlen_q, p->Max_seqlen_k, p->varlen_type,
                        p->causal_type, p->dropout_p, p->philox_seed_ptr, &s);
   if (e != FA_SUCCESS) return e;
-  if ((e = check_act(p->Out, p->Q.dtype)) != FA_SUCCESS) return e;
+  bool pieces = !s.elementwise;
+  if ((e = check_act(p->Out, p->Q.dtype, &pieces)) != FA_SUCCESS) return e;
+  s.elementwise = !pieces;
   for (int i = 0; i < 4; ++i)
     if (p->Out.sizes[i] != (i == 3 ? p->V.sizes[3] : p->Q.sizes[i])) return FA_ERROR_INVALID_VALUE;
   if (p->A.ptr != nullptr) return FA_ERROR_NOT_SUPPORTED;   // alibi: USE_ALIBI=false in attn_fwd.cc:123
@@ -275,11 +285,13 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
                        p->causal_type, p->dropout_p, p->philox_seed_ptr, &s);
   if (e != FA_SUCCESS) return e;
   const int dt = p->Q.dtype;
-  if ((e = check_act(p->Out, dt)) != FA_SUCCESS) return e;
-  if ((e = check_act(p->DO, dt)) != FA_SUCCESS) return e;
-  if ((e = check_act(p->DQ, dt)) != FA_SUCCESS) return e;
-  if ((e = check_act(p->DK, dt)) != FA_SUCCESS) return e;
-  if ((e = check_act(p->DV, dt)) != FA_SUCCESS) return e;
+  bool pieces = !s.elementwise;
+  if ((e = check_act(p->Out, dt, &pieces)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DO, dt, &pieces)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DQ, dt, &pieces)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DK, dt, &pieces)) != FA_SUCCESS) return e;
+  if ((e = check_act(p->DV, dt, &pieces)) != FA_SUCCESS) return e;
+  s.elementwise = !pieces;
   for (int i = 0; i < 4; ++i) {
     const auto o_i = i == 3 ? p->V.sizes[3] : p->Q.sizes[i];
     if (p->Out.sizes[i] != o_i || p->DO.sizes[i] != o_i ||
@@ -299,8 +311,8 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   }
   int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2
-  if (be == 1 && (!is_16bit(dt) || s.d > 256)) {
-    // the vector-ALU kernels (fp32, head dims above 256) exist for the split backend only: a forced fused backend cannot take the input, an
+  if (be == 1 && (!is_16bit(dt) || s.d > 256 || s.elementwise)) {
+    // the vector-ALU kernels (fp32, head dims above 256, element-wise rows) exist for the split backend only: a forced fused backend cannot take the input, an
     // unforced choice falls back to split when a delta buffer is there (template/op.cc:57-70)
     const bool forced = opt != nullptr && opt->force_backend_index >= 0;
     if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
@@ -316,6 +328,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 }
 
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
+  if (s.elementwise) return fa::run_fwd_valu(dtype, d, a, stream);
   if (dtype == FA_DTYPE_FLOAT32)
     return d <= 256 ? fa::run_fwd_f32(d, a, s.windowed, s.bias, s.dropout, stream) : fa::run_fwd_valu(dtype, d, a, stream);
   if (d > 256) return fa::run_fwd_d512(dtype, a, s.windowed, s.bias, s.dropout, stream);
@@ -409,8 +422,9 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
   if (e != FA_SUCCESS) return e;
   // the vector-ALU kernels (fp32) and the split-head-dim kernels (above 256): 32 rows per workgroup, 3-D grid
-  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;
-  const fa::TileShape t = params->Q.dtype == FA_DTYPE_FLOAT32
+  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256 || s.elementwise;
+  const fa::TileShape t = s.elementwise ? fa::TileShape{32, 1, 4, 0}
+                          : params->Q.dtype == FA_DTYPE_FLOAT32
                               ? (s.d <= 256 ? fa::f32_tile_shape(s.d, -1) : fa::TileShape{32, 1, 4, 0})
                           : s.d > 256 ? fa::d512_tile_shape(-1)
                                       : fa::fwd_tile_shape(params->Q.dtype, s.d, s.windowed);
@@ -419,7 +433,7 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   if (valu) {
     const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
     const int mt = (s.max_sq + t.block_m - 1) / t.block_m;
-    if (params->Q.dtype == FA_DTYPE_FLOAT32 && s.d > 256) {      // vector-ALU kernels: 3-D grid
+    if (s.elementwise || (params->Q.dtype == FA_DTYPE_FLOAT32 && s.d > 256)) {      // vector-ALU kernels: 3-D grid
       out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz;
     } else {      // one workgroup per tile, the tiles of a kv-head's group back to back on one XCD
       out->grid[0] = fa::kNumXcd * ((nz * s.hk + fa::kNumXcd - 1) / fa::kNumXcd) * (s.hq / s.hk) * mt;
@@ -452,10 +466,10 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   int be = 0;
   int e = validate_bwd(params, FA_BWD_PARAMS_VERSION, options, &s, &be);
   if (e != FA_SUCCESS) return e;
-  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256;   // vector-ALU kernels: 32 rows per workgroup
+  const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256 || s.elementwise;   // vector-ALU kernels: 32 rows per workgroup
   if (valu && kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
-  const bool split_d = params->Q.dtype != FA_DTYPE_FLOAT32 && s.d > 256 && kernel_slot != 0;
-  const bool f32_mfma = params->Q.dtype == FA_DTYPE_FLOAT32 && s.d <= 256 && kernel_slot != 0;
+  const bool split_d = !s.elementwise && params->Q.dtype != FA_DTYPE_FLOAT32 && s.d > 256 && kernel_slot != 0;
+  const bool f32_mfma = !s.elementwise && params->Q.dtype == FA_DTYPE_FLOAT32 && s.d <= 256 && kernel_slot != 0;
   const fa::TileShape t = f32_mfma ? fa::f32_tile_shape(s.d, kernel_slot)
                           : split_d ? fa::d512_tile_shape(kernel_slot)
                           : valu  ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
@@ -537,6 +551,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
     a.sb_m = (int64_t)p->B.strides[2]; a.sb_n = (int64_t)p->B.strides[3];
   }
   a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_qk; a.head_dim_v = s.d_v;
+  a.elementwise = s.elementwise ? 1 : 0;
   a.sm_scale = p->Sm_scale;
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
@@ -546,7 +561,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
   a.atomic_counter = static_cast<int32_t*>(p->persistent_atomic_counter.ptr);
   a.num_cu = dev->num_cu;
 
-  const fa::TileShape t = (p->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256) ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(p->Q.dtype, s.d, s.windowed);
+  const fa::TileShape t = (p->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256 || s.elementwise) ? fa::TileShape{32, 1, 4, 0} : fa::fwd_tile_shape(p->Q.dtype, s.d, s.windowed);
   FA_LOG(4, "attn_fwd: D=%d BLOCK_M=%d BLOCK_N=%d waves=%d lds=%d windowed=%d bias=%d dropout=%d nseq=%d",
          s.d, t.block_m, t.block_n, t.num_waves, t.lds_bytes, (int)s.windowed, (int)s.bias,
          (int)s.dropout, s.num_seqlens);
@@ -629,6 +644,7 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     a.sdb_m = (int64_t)p->DB.strides[2]; a.sdb_n = (int64_t)p->DB.strides[3];
   }
   a.batch = s.batch; a.hq = s.hq; a.hk = s.hk; a.head_dim = s.d_qk; a.head_dim_v = s.d_v;
+  a.elementwise = s.elementwise ? 1 : 0;
   a.sm_scale = p->Sm_scale;
   a.seq = seq_args(s, p->cu_seqlens_q, p->cu_seqlens_k, p->seq_strides_q, p->seq_strides_k, p->varlen_type);
   a.mask = fa::MaskArgs{p->causal_type, p->window_left, p->window_right};
@@ -654,20 +670,23 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       }
     }
     a.delta = static_cast<float*>(delta.ptr);
-    const bool f32 = dt == FA_DTYPE_FLOAT32;      // fp32 MFMA kernels up to head dim 256, vector-ALU kernels above
-    const bool big = !f32 && s.d > 256;           // head dim split over the waves
+    const bool slow = s.elementwise;              // rows moved element by element: vector-ALU kernels
+    const bool f32 = !slow && dt == FA_DTYPE_FLOAT32;      // fp32 MFMA kernels up to head dim 256, vector-ALU kernels above
+    const bool big = !slow && !f32 && s.d > 256;  // head dim split over the waves
     // fp32 and the head dims above 256 take delta from the vector-ALU kernel.  The dQ kernel of the
     // 16-bit types up to head dim 256 computes delta from the O and dO rows it holds and writes it
     // out; the dK/dV kernel runs after it and reads it, so the whole backward is two launches
     // (kernel_slot 0 still launches the preprocess kernel on its own).
-    const bool delta_launch = f32 || big;
+    const bool delta_launch = f32 || big || slow;
     if (kernel_slot == 0 || (kernel_slot < 0 && delta_launch))
       err = delta_launch ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
     const int order[2] = {delta_launch ? 1 : 2, delta_launch ? 2 : 1};
     for (int i = 0; i < 2 && err == hipSuccess; ++i) {
       const int slot = order[i];
       if (kernel_slot >= 0 && kernel_slot != slot) continue;
-      if (f32)
+      if (slow)
+        err = fa::run_bwd_valu(dt, s.d, slot, a, stream);
+      else if (f32)
         err = s.d <= 256 ? fa::run_bwd_f32(s.d, slot, a, s.windowed, s.bias, s.dropout, stream)
                          : fa::run_bwd_valu(dt, s.d, slot, a, stream);
       else if (big)

@@ -40,8 +40,9 @@ struct FwdArgs {
   Strides3 sq, sk, sv, so;
   int64_t sb_z, sb_h, sb_m, sb_n;
   int32_t batch, hq, hk;
-  int32_t head_dim;      // columns of Q and K (<= the compiled head dim, multiple of 8)
+  int32_t head_dim;      // columns of Q and K (<= the compiled head dim; a multiple of 8 unless `elementwise`)
   int32_t head_dim_v;    // columns of V, Out and dOut (same bounds)
+  int32_t elementwise;   // rows are not made of aligned 16-byte pieces: the vector-ALU kernels move single elements
   float sm_scale;
   SeqArgs seq;
   MaskArgs mask;
@@ -65,8 +66,9 @@ struct BwdArgs {
   int64_t sb_z, sb_h, sb_m, sb_n;
   int64_t sdb_z, sdb_h, sdb_m, sdb_n;
   int32_t batch, hq, hk;
-  int32_t head_dim;      // columns of Q and K (<= the compiled head dim, multiple of 8)
+  int32_t head_dim;      // columns of Q and K (<= the compiled head dim; a multiple of 8 unless `elementwise`)
   int32_t head_dim_v;    // columns of V, Out and dOut (same bounds)
+  int32_t elementwise;   // rows are not made of aligned 16-byte pieces: the vector-ALU kernels move single elements
   float sm_scale;
   SeqArgs seq;
   MaskArgs mask;

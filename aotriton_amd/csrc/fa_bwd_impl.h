@@ -1299,6 +1299,13 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 // ---------------------------------------------------------------------------
 // Kernels
 // ---------------------------------------------------------------------------
+// Whether the dK/dV kernel walks the level list: persistent workgroups over sequences of different
+// lengths, few enough (sequence, kv-head) entries per XCD for the table.
+template <int D>
+__host__ __device__ inline bool dkdv_level_list(const BwdArgs& a) {
+  return D < 256 && a.seq.num_seqlens != 0 && a.bias == nullptr && a.zh_per_xcd <= kLevelCap && a.num_n_tiles <= 0xffff;
+}
+
 template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kPad>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dkdv_kernel(const BwdArgs a) {
@@ -1417,13 +1424,6 @@ inline int bwd_nseq(const BwdArgs& a) {
 // grid was 10 % slower, while it gains 1 % at the headline shape and 12 % on packed
 // sequences of very different lengths.  D = 256 also gets one workgroup per item: its
 // dK/dV kernel has no register to spare for the loop.
-// Whether the dK/dV kernel walks the level list: persistent workgroups over sequences of different
-// lengths, few enough (sequence, kv-head) entries per XCD for the table.
-template <int D>
-__host__ __device__ inline bool dkdv_level_list(const BwdArgs& a) {
-  return D < 256 && a.seq.num_seqlens != 0 && a.bias == nullptr && a.zh_per_xcd <= kLevelCap && a.num_n_tiles <= 0xffff;
-}
-
 template <int D>
 inline int persistent_workers(const BwdArgs& a) {
   if (a.bias != nullptr || D >= 256) return a.items_per_xcd;

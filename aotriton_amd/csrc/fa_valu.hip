@@ -34,15 +34,20 @@ template <> struct Quad<float> { using type = f32x4; };
 template <typename T> __device__ __forceinline__ T from_float(float x) { return Traits<T>::cvt(x); }
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
 
-// columns [0, cols) of a row of D = 8*DPL elements as floats; the rest reads as zero
+// columns [0, cols) of a row of D = 8*DPL elements as floats; the rest reads as zero.  `elem`: the
+// row is not made of aligned groups of four (a head dim that is no multiple of 8, odd strides, a
+// base that is only element-aligned) and is read element by element.
 template <int DPL, typename T>
-__device__ __forceinline__ Row<DPL> load_row(const T* p, int sub, int cols, bool ok) {
+__device__ __forceinline__ Row<DPL> load_row(const T* p, int sub, int cols, bool ok, bool elem) {
   using quad = typename Quad<T>::type;
   Row<DPL> r;
 #pragma unroll
   for (int j = 0; j < DPL / 4; ++j) {
     const int c = 4 * sub + 32 * j;
-    if (ok && c < cols) {
+    if (elem) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r.x[4 * j + e] = ok && c + e < cols ? (float)p[c + e] : 0.f;
+    } else if (ok && c < cols) {
       const quad v = *reinterpret_cast<const quad*>(p + c);
 #pragma unroll
       for (int e = 0; e < 4; ++e) r.x[4 * j + e] = (float)v[e];
@@ -55,12 +60,16 @@ __device__ __forceinline__ Row<DPL> load_row(const T* p, int sub, int cols, bool
 }
 
 template <int DPL, typename T>
-__device__ __forceinline__ void store_row(T* p, const Row<DPL>& r, int sub, int cols, float scale) {
+__device__ __forceinline__ void store_row(T* p, const Row<DPL>& r, int sub, int cols, float scale, bool elem) {
   using quad = typename Quad<T>::type;
 #pragma unroll
   for (int j = 0; j < DPL / 4; ++j) {
     const int c = 4 * sub + 32 * j;
-    if (c < cols) {
+    if (elem) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c + e < cols) p[c + e] = from_float<T>(r.x[4 * j + e] * scale);
+    } else if (c < cols) {
       quad v;
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = from_float<T>(r.x[4 * j + e] * scale);
@@ -129,7 +138,7 @@ __global__ void valu_fwd_kernel(const FwdArgs a) {
   const T* bp = a.bias ? reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z +
                                  (int64_t)h * a.sb_h + (int64_t)mc * a.sb_m
                            : nullptr;
-  const Row<DPL> q = load_row<DPL, T>(qp, sub, a.head_dim, true);
+  const Row<DPL> q = load_row<DPL, T>(qp, sub, a.head_dim, true, a.elementwise != 0);
   Row<DPL> o;
 #pragma unroll
   for (int e = 0; e < DPL; ++e) o.x[e] = 0.f;
@@ -144,7 +153,7 @@ __global__ void valu_fwd_kernel(const FwdArgs a) {
     n_hi = m_last + vis.right < n_hi ? m_last + vis.right : n_hi;
   }
   for (int n = n_lo; n <= n_hi; ++n) {
-    const Row<DPL> kr = load_row<DPL, T>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true);
+    const Row<DPL> kr = load_row<DPL, T>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true, a.elementwise != 0);
     float s = dot8<DPL>(q, kr) * qk_scale;                                   // fwd_kernel_inner.py:166
     if (bp) s += (float)bp[(int64_t)n * a.sb_n] * kLog2e;                           // :187
     if (!vis(m, n) || s == -__builtin_inff()) continue;                      // lanes of a row agree
@@ -155,7 +164,7 @@ __global__ void valu_fwd_kernel(const FwdArgs a) {
     mi = m_new;
     const bool keep = !dropout || dropout_keep1(ds, m, n);
     const float pv = keep ? p : 0.f;
-    const Row<DPL> vr = load_row<DPL, T>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true);
+    const Row<DPL> vr = load_row<DPL, T>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true, a.elementwise != 0);
 #pragma unroll
     for (int e = 0; e < DPL; ++e) o.x[e] = __builtin_fmaf(pv, vr.x[e], o.x[e] * alpha);
   }
@@ -165,7 +174,7 @@ __global__ void valu_fwd_kernel(const FwdArgs a) {
   if (dropout) inv *= ds.scale;                                              // fwd_kernel.py:573-580
   T* op = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
               (int64_t)(si.q_start + m) * a.so.s;
-  store_row<DPL, T>(op, o, sub, a.head_dim_v, inv);
+  store_row<DPL, T>(op, o, sub, a.head_dim_v, inv, a.elementwise != 0);
   if (a.lse && sub == 0)
     a.lse[lse_offset(si, h, a.hq) + m] = alive ? (mi + fast_log2(li)) * kLn2 : __builtin_inff();   // :610-612, :327-355
 }
@@ -184,7 +193,8 @@ __global__ void valu_delta_kernel(const BwdArgs a) {
                     (int64_t)(si.q_start + mc) * a.so.s;
   const T* dop = reinterpret_cast<const T*>(a.dout) + (int64_t)si.batch_index * a.sdo.z +
                      (int64_t)h * a.sdo.h + (int64_t)(si.q_start + mc) * a.sdo.s;
-  const float d = dot8<DPL>(load_row<DPL, T>(op, sub, a.head_dim_v, true), load_row<DPL, T>(dop, sub, a.head_dim_v, true));
+  const bool elem = a.elementwise != 0;
+  const float d = dot8<DPL>(load_row<DPL, T>(op, sub, a.head_dim_v, true, elem), load_row<DPL, T>(dop, sub, a.head_dim_v, true, elem));
   if (row_ok && sub == 0) a.delta[lse_offset(si, h, a.hq) + m] = d;
 }
 
@@ -216,8 +226,8 @@ __global__ void valu_dq_kernel(const BwdArgs a) {
   T* dbp = a.db ? reinterpret_cast<T*>(a.db) + (int64_t)si.batch_index * a.sdb_z + (int64_t)h * a.sdb_h +
                           (int64_t)mc * a.sdb_m
                     : nullptr;
-  const Row<DPL> q = load_row<DPL, T>(reinterpret_cast<const T*>(a.q) + qoff, sub, a.head_dim, true);
-  const Row<DPL> dout = load_row<DPL, T>(dop, sub, a.head_dim_v, true);
+  const Row<DPL> q = load_row<DPL, T>(reinterpret_cast<const T*>(a.q) + qoff, sub, a.head_dim, true, a.elementwise != 0);
+  const Row<DPL> dout = load_row<DPL, T>(dop, sub, a.head_dim_v, true, a.elementwise != 0);
   const int64_t lo = lse_offset(si, h, a.hq) + mc;
   const float L = a.lse[lo] * kRcpLn2;                                       // bwd_kernel_dq.py:305
   const float delta = a.delta[lo];
@@ -228,8 +238,8 @@ __global__ void valu_dq_kernel(const BwdArgs a) {
   for (int n = 0; n < si.seqlen_k; ++n) {
     float dsv = 0.f;
     if (vis(m, n)) {
-      const Row<DPL> kr = load_row<DPL, T>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true);
-      const Row<DPL> vr = load_row<DPL, T>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true);
+      const Row<DPL> kr = load_row<DPL, T>(kb + (int64_t)n * a.sk.s, sub, a.head_dim, true, a.elementwise != 0);
+      const Row<DPL> vr = load_row<DPL, T>(vb + (int64_t)n * a.sv.s, sub, a.head_dim_v, true, a.elementwise != 0);
       float x = dot8<DPL>(q, kr) * qk_scale;
       if (bp) x += (float)bp[(int64_t)n * a.sb_n] * kLog2e;
       const float p = fast_exp2(x - L);                                      // bwd_inner_dq.py:158-160
@@ -244,7 +254,7 @@ __global__ void valu_dq_kernel(const BwdArgs a) {
   if (!row_ok) return;
   T* dqp = reinterpret_cast<T*>(a.dq) + (int64_t)si.batch_index * a.sdq.z + (int64_t)h * a.sdq.h +
                (int64_t)(si.q_start + m) * a.sdq.s;
-  store_row<DPL, T>(dqp, dq, sub, a.head_dim, a.sm_scale);                      // bwd_kernel_dq.py:374-376
+  store_row<DPL, T>(dqp, dq, sub, a.head_dim, a.sm_scale, a.elementwise != 0);                      // bwd_kernel_dq.py:374-376
 }
 
 // One row of K per lane group, all q-heads of its group and all queries: dK and dV.
@@ -262,10 +272,10 @@ __global__ void valu_dkdv_kernel(const BwdArgs a) {
   const int group = a.hq / a.hk;
   const Row<DPL> kr = load_row<DPL, T>(reinterpret_cast<const T*>(a.k) + (int64_t)si.batch_index * a.sk.z +
                                         (int64_t)hk * a.sk.h + (int64_t)(si.k_start + nc) * a.sk.s,
-                                    sub, a.head_dim, true);
+                                    sub, a.head_dim, true, a.elementwise != 0);
   const Row<DPL> vr = load_row<DPL, T>(reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z +
                                         (int64_t)hk * a.sv.h + (int64_t)(si.k_start + nc) * a.sv.s,
-                                    sub, a.head_dim_v, true);
+                                    sub, a.head_dim_v, true, a.elementwise != 0);
   const float qk_scale = a.sm_scale * kLog2e;
   Row<DPL> dk, dv;
 #pragma unroll
@@ -284,8 +294,8 @@ __global__ void valu_dkdv_kernel(const BwdArgs a) {
     const int64_t lo = lse_offset(si, h, a.hq);
     for (int m = 0; m < si.seqlen_q; ++m) {
       if (!vis(m, n)) continue;                                              // lanes of a row agree
-      const Row<DPL> qr = load_row<DPL, T>(qb + (int64_t)m * a.sq.s, sub, a.head_dim, true);
-      const Row<DPL> dor = load_row<DPL, T>(dob + (int64_t)m * a.sdo.s, sub, a.head_dim_v, true);
+      const Row<DPL> qr = load_row<DPL, T>(qb + (int64_t)m * a.sq.s, sub, a.head_dim, true, a.elementwise != 0);
+      const Row<DPL> dor = load_row<DPL, T>(dob + (int64_t)m * a.sdo.s, sub, a.head_dim_v, true, a.elementwise != 0);
       float x = dot8<DPL>(qr, kr) * qk_scale;
       if (bb) x += (float)bb[(int64_t)m * a.sb_m] * kLog2e;
       const float p = fast_exp2(x - a.lse[lo + m] * kRcpLn2);               // bwd_inner_dk_dv.py:185-188
@@ -306,32 +316,59 @@ __global__ void valu_dkdv_kernel(const BwdArgs a) {
                (int64_t)(si.k_start + n) * a.sdk.s;
   T* dvp = reinterpret_cast<T*>(a.dv) + (int64_t)si.batch_index * a.sdv.z + (int64_t)hk * a.sdv.h +
                (int64_t)(si.k_start + n) * a.sdv.s;
-  store_row<DPL, T>(dkp, dk, sub, a.head_dim, a.sm_scale);                      // bwd_kernel_dk_dv.py:387-389
-  store_row<DPL, T>(dvp, dv, sub, a.head_dim_v, 1.0f);
+  store_row<DPL, T>(dkp, dk, sub, a.head_dim, a.sm_scale, a.elementwise != 0);                      // bwd_kernel_dk_dv.py:387-389
+  store_row<DPL, T>(dvp, dv, sub, a.head_dim_v, 1.0f, a.elementwise != 0);
 }
+
+// head_dim: 64, 128, 256 or 512, the one that holds the tensors' head dims.  The 16-bit types are
+// built for 128, 256 and 512 (the MFMA kernels serve them wherever rows are made of aligned 16-byte
+// pieces; what is left are the element-wise cases, and 64 columns run on the 128 build).
+template <template <typename, int> class Launch, typename... A>
+hipError_t valu_dispatch(int dtype, int head_dim, A&&... args) {
+  if (dtype == kDtypeF32) {
+    switch (head_dim) {
+      case 64: return Launch<float, 8>::run(args...);
+      case 128: return Launch<float, 16>::run(args...);
+      case 256: return Launch<float, 32>::run(args...);
+      case 512: return Launch<float, 64>::run(args...);
+    }
+    return hipErrorNotSupported;
+  }
+  if (dtype != kDtypeBF16 && dtype != kDtypeF16) return hipErrorNotSupported;
+  const bool bf = dtype == kDtypeBF16;
+  switch (head_dim) {
+    case 64:
+    case 128: return bf ? Launch<bf16_t, 16>::run(args...) : Launch<f16_t, 16>::run(args...);
+    case 256: return bf ? Launch<bf16_t, 32>::run(args...) : Launch<f16_t, 32>::run(args...);
+    case 512: return bf ? Launch<bf16_t, 64>::run(args...) : Launch<f16_t, 64>::run(args...);
+  }
+  return hipErrorNotSupported;
+}
+
+template <typename T, int DPL> struct LaunchFwd {
+  static hipError_t run(const dim3& grid, const FwdArgs& a, hipStream_t s) {
+    hipLaunchKernelGGL((valu_fwd_kernel<T, DPL>), grid, dim3(256), 0, s, a);
+    return hipGetLastError();
+  }
+};
+template <typename T, int DPL> struct LaunchBwd {
+  static hipError_t run(int kernel_slot, const dim3& gq, const dim3& gk, const BwdArgs& a, hipStream_t s) {
+    switch (kernel_slot) {
+      case 0: hipLaunchKernelGGL((valu_delta_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;
+      case 1: hipLaunchKernelGGL((valu_dkdv_kernel<T, DPL>), gk, dim3(256), 0, s, a); break;
+      case 2: hipLaunchKernelGGL((valu_dq_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;
+      default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+  }
+};
 
 }  // namespace
 
-// head_dim: 64, 128, 256 or 512, the one that holds the tensors' head dims.  The 16-bit types
-// are built for 512 only (the MFMA kernels serve the others).
 hipError_t run_fwd_valu(int dtype, int head_dim, const FwdArgs& a, hipStream_t s) {
   const dim3 grid((a.seq.max_seqlen_q + kRowsPerBlock - 1) / kRowsPerBlock, a.hq, nseq_of(a.seq, a.batch));
   if (grid.x == 0 || grid.z == 0) return hipSuccess;      // an empty tensor: nothing to write
-  if (dtype == kDtypeF32) {
-    switch (head_dim) {
-      case 64: hipLaunchKernelGGL((valu_fwd_kernel<float, 8>), grid, dim3(256), 0, s, a); break;
-      case 128: hipLaunchKernelGGL((valu_fwd_kernel<float, 16>), grid, dim3(256), 0, s, a); break;
-      case 256: hipLaunchKernelGGL((valu_fwd_kernel<float, 32>), grid, dim3(256), 0, s, a); break;
-      case 512: hipLaunchKernelGGL((valu_fwd_kernel<float, 64>), grid, dim3(256), 0, s, a); break;
-      default: return hipErrorNotSupported;
-    }
-  } else if (head_dim == 512) {
-    if (dtype == kDtypeBF16) hipLaunchKernelGGL((valu_fwd_kernel<bf16_t, 64>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((valu_fwd_kernel<f16_t, 64>), grid, dim3(256), 0, s, a);
-  } else {
-    return hipErrorNotSupported;
-  }
-  return hipGetLastError();
+  return valu_dispatch<LaunchFwd>(dtype, head_dim, grid, a, s);
 }
 
 // kernel_slot: 0 delta, 1 dK/dV, 2 dQ (and dB)
@@ -341,28 +378,7 @@ hipError_t run_bwd_valu(int dtype, int head_dim, int kernel_slot, const BwdArgs&
   const dim3 gk((a.seq.max_seqlen_k + kRowsPerBlock - 1) / kRowsPerBlock, a.hk, nseq);
   const dim3& g = kernel_slot == 1 ? gk : gq;
   if (g.x == 0 || g.z == 0) return hipSuccess;            // an empty tensor: nothing to write
-#define FA_VALU_LAUNCH(T, DPL)                                                                     \
-  switch (kernel_slot) {                                                                           \
-    case 0: hipLaunchKernelGGL((valu_delta_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;        \
-    case 1: hipLaunchKernelGGL((valu_dkdv_kernel<T, DPL>), gk, dim3(256), 0, s, a); break;         \
-    case 2: hipLaunchKernelGGL((valu_dq_kernel<T, DPL>), gq, dim3(256), 0, s, a); break;           \
-    default: return hipErrorInvalidValue;                                                          \
-  }
-  if (dtype == kDtypeF32) {
-    switch (head_dim) {
-      case 64: FA_VALU_LAUNCH(float, 8) break;
-      case 128: FA_VALU_LAUNCH(float, 16) break;
-      case 256: FA_VALU_LAUNCH(float, 32) break;
-      case 512: FA_VALU_LAUNCH(float, 64) break;
-      default: return hipErrorNotSupported;
-    }
-  } else if (head_dim == 512) {
-    if (dtype == kDtypeBF16) { FA_VALU_LAUNCH(bf16_t, 64) } else { FA_VALU_LAUNCH(f16_t, 64) }
-  } else {
-    return hipErrorNotSupported;
-  }
-#undef FA_VALU_LAUNCH
-  return hipGetLastError();
+  return valu_dispatch<LaunchBwd>(dtype, head_dim, kernel_slot, gq, gk, a, s);
 }
 
 }  // namespace fa

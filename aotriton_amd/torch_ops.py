@@ -175,7 +175,7 @@ def _routable(query, key, value, attn_mask, dropout_p):
     if not (key.dtype == query.dtype and value.dtype == query.dtype):
         return False
     dqk, dv = query.shape[-1], value.shape[-1]
-    if dqk % 8 or dv % 8 or dqk > 512 or dv > 512 or key.shape[-1] != dqk:
+    if dqk > 512 or dv > 512 or key.shape[-1] != dqk:
         return False
     if query.shape[1] % max(key.shape[1], 1) or key.shape[1] != value.shape[1]:
         return False

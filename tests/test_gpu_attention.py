@@ -338,6 +338,53 @@ def test_sampled_strides_bias_layouts_and_masks(i):
         check('db', bg.grad, rg[3], lg[3], FUDGE['db'])
 
 
+@pytest.mark.parametrize('D', [7, 23, 37, 53, 67, 73, 89, 113, 149, 179, 211, 241, 203, 300, 509])
+def test_head_dims_that_are_no_multiple_of_8(D):
+    """The reference rounds ANY head dim up to a compiled one and masks the excess columns
+    (modules/flash/csrc/attn_fwd.cc:76-82,109); its test grid includes the primes below
+    (modules/flash/tests/test_forward.py:22,92).  Rows of such tensors are not made of aligned 16-byte
+    pieces and run on the kernels that move single elements (split backend)."""
+    dtype = [torch.bfloat16, torch.float16, torch.float32][D % 3]
+    causal = [False, True, (9, 4)][(D // 3) % 3]
+    _run_case(2, 4, 2, 70, 83, D, dtype, causal, dropout_p=0.2 if D % 2 else 0.0, bias=D % 5 == 0, bwd_backend=0, seed=D)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('how', ['base', 'row_stride', 'head_stride'])
+def test_rows_that_are_not_16_byte_aligned(dtype, how):
+    """Head dim 64, but a base address that is only element-aligned, a row stride of 65 or a head stride
+    that is no multiple of 8: the same element-wise kernels, same results as the oracle."""
+    from aotriton_amd import flash
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from oracle import fa_ref
+    B, Hq, Hk, Sq, Sk, D = 2, 2, 2, 45, 61, 64
+    g = torch.Generator().manual_seed(3)
+    def mk(H, S):
+        if how == 'base':
+            return torch.randn(B * H * S * D + 1, generator=g).to(dtype).to(DEV)[1:].view(B, H, S, D)
+        if how == 'row_stride':
+            return torch.randn(B, H, S, D + 1, generator=g).to(dtype).to(DEV)[..., :D]
+        return torch.randn(B, H, S * D + 3, generator=g).to(dtype).to(DEV)[..., :S * D].view(B, H, S, D)
+    q, k, v, do = mk(Hq, Sq), mk(Hk, Sk), mk(Hk, Sk), mk(Hq, Sq)
+    sm = D ** -0.5
+    ext = AttentionExtraArgs(return_logsumexp=True, fillnan=True, bwd_backend=0)
+    qg, kg, vg = [t.detach().requires_grad_() for t in (q, k, v)]
+    o, _, L = attention(qg, kg, vg, None, True, sm, 0.0, ext)
+    o.backward(do)
+    torch.cuda.synchronize()
+    ct, wl, wr = flash.translate_causal(True)
+    hp = torch.float64 if dtype == torch.float32 else torch.float32
+    f = lambda t: t.to(hp)
+    ro, rl, _ = fa_ref.attn_fwd_ref(f(q), f(k), f(v), None, sm, ct, wl, wr, 0.0, None)
+    lo, ll, _ = fa_ref.attn_fwd_ref(q, k, v, None, sm, ct, wl, wr, 0.0, None)
+    check('out', o, ro, lo, FUDGE['out'])
+    rg = fa_ref.attn_bwd_ref(f(q), f(k), f(v), None, sm, ro, f(do), rl, ct, wl, wr, 0.0, None)
+    lg = fa_ref.attn_bwd_ref(q, k, v, None, sm, lo, do, ll.to(q.dtype), ct, wl, wr, 0.0, None)
+    check('dq', qg.grad, rg[0], lg[0], FUDGE['dq'])
+    check('dk', kg.grad, rg[1], lg[1], FUDGE['dk'])
+    check('dv', vg.grad, rg[2], lg[2], FUDGE['dv'])
+
+
 @pytest.mark.parametrize('dtype,D', [(torch.bfloat16, 64), (torch.float16, 128), (torch.bfloat16, 256), (torch.bfloat16, 512),
                                      (torch.float32, 128), (torch.float32, 320), (torch.bfloat16, 72)])
 @pytest.mark.parametrize('causal', [False, True])

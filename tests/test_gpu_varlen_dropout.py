@@ -134,6 +134,12 @@ def test_many_packed_sequences(nseq, hk, causal):
     _run_varlen_case(lens, lens, 2 * hk, hk, 64, torch.bfloat16, causal, 0)
 
 
+@pytest.mark.parametrize('D,dtype', [(37, torch.bfloat16), (203, torch.float16), (7, torch.float32)])
+def test_compact_varlen_head_dim_no_multiple_of_8(D, dtype):
+    # packed sequences on the element-wise kernels (any head dim, modules/flash/csrc/attn_fwd.cc:76-82)
+    _run_varlen_case([5, 0, 70, 33], [9, 64, 41, 33], 4, 2, D, dtype, True, 0, p=0.1)
+
+
 def _sampled_varlen_cases(n=40, seed=4242):
     """Seeded packed-sequence cases: 1-6 sequences of 0-300 tokens (the reference draws its
     lengths from a fixed list, tests/test_varlen.py:34-47), key lengths that differ from the

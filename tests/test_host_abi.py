@@ -116,9 +116,13 @@ def test_validate_fwd_error_contract():
     p7, k7 = _fwd_params(D=512)                                                # above 256: the head dim split over the waves, 64 rows per workgroup
     err, cfg = query_fwd_config(p7)
     assert err == E.hipSuccess and cfg.head_dim == 512 and cfg.block_m == 64 and list(cfg.grid) == [16, 1, 1]
-    for bad in (520, 100):                                                     # > 512, or rows not a multiple of 16 bytes
-        pb, kb = _fwd_params(D=bad)
-        assert validate_fwd(pb, 3) == E.hipErrorNotSupported
+    pb, kb = _fwd_params(D=520)                                                # above 512
+    assert validate_fwd(pb, 3) == E.hipErrorNotSupported
+    for odd in (100, 7, 203):                                                  # rows that are not made of 16-byte pieces: element-wise kernels
+        po, ko = _fwd_params(D=odd)
+        err, cfg = query_fwd_config(po)
+        assert err == E.hipSuccess and cfg.head_dim == {100: 128, 7: 64, 203: 256}[odd] and cfg.block_m == 32
+        assert list(cfg.grid)[1:] == [po.Q.sizes[1], po.Q.sizes[0]]
     p3, k3 = _fwd_params(dtype=torch.float32)
     assert validate_fwd(p3, 3) == E.hipSuccess                                 # fp32: fp32 MFMA kernels
     p4, k4 = _fwd_params(Hq=5, Hk=2)

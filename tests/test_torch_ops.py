@@ -188,6 +188,25 @@ def test_router_leaves_cpu_calls_to_torch():
 
 
 @pytest.mark.gpu
+def test_sdpa_head_dim_that_is_no_multiple_of_8():
+    """Any head dim up to 512 is taken (the reference pads it, modules/flash/csrc/attn_fwd.cc:76-82); against
+    torch's math backend."""
+    import torch.nn.functional as F
+    from aotriton_amd import torch_ops
+    q, k, v, _, do = _inputs(B=2, Hq=4, Hk=4, Sq=90, Sk=90, D=37)
+    req = lambda t: t.detach().clone().requires_grad_()
+    a, b, c = req(q), req(k), req(v)
+    o = torch_ops.scaled_dot_product_attention(a, b, c, is_causal=True)
+    o.backward(do)
+    a2, b2, c2 = req(q.float()), req(k.float()), req(v.float())
+    with torch.nn.attention.sdpa_kernel(torch.nn.attention.SDPBackend.MATH):
+        o2 = F.scaled_dot_product_attention(a2, b2, c2, is_causal=True)
+    o2.backward(do.float())
+    for x, y in ((o, o2), (a.grad, a2.grad), (b.grad, b2.grad), (c.grad, c2.grad)):
+        assert (x.float() - y).abs().max().item() < 6e-2
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize('hook', ['mode', 'install'])
 def test_f_sdpa_routes_to_the_library(hook):
     """F.scaled_dot_product_attention itself, unchanged call sites: under the router the library's
