@@ -213,7 +213,10 @@ int check_common(const fa_tensor4& Q, const fa_tensor4& K, const fa_tensor4& V, 
   s.bias = B.ptr != nullptr;      // attn_fwd.cc:122
   if (s.bias) {
     if (B.dtype != dtype) return FA_ERROR_INVALID_VALUE;
-    if (s.num_seqlens != 0) return FA_ERROR_NOT_SUPPORTED;   // bias has no packed layout
+    // Sequences of a varlen batch index the bias like the reference's kernels do
+    // (modules/flash/kernel/fwd_kernel.py:393-395): batch stride times the batch index, which is the
+    // sequence for the padded layout and 0 for packed tokens (one bias shared by all sequences), rows
+    // and columns counted from the sequence's start; hence sizes (batch of Q, Hq, Max_seqlen_q, Max_seqlen_k).
     if ((int)B.sizes[0] != s.batch || (int)B.sizes[1] != s.hq || (int)B.sizes[2] != s.max_sq ||
         (int)B.sizes[3] != s.max_sk)
       return FA_ERROR_INVALID_VALUE;
@@ -305,6 +308,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   if (p->L.ptr != nullptr && (e = check_row_stats(p->L, s.row_stats)) != FA_SUCCESS) return e;
   if (p->DB.ptr != nullptr) {
     if (!s.bias) return FA_ERROR_INVALID_VALUE;
+    if (s.num_seqlens > 0) return FA_ERROR_NOT_SUPPORTED;   // packed tokens share one bias: every sequence would write the same dB rows
     if (p->DB.dtype != dt) return FA_ERROR_INVALID_VALUE;
     for (int i = 0; i < 4; ++i)
       if (p->DB.sizes[i] != p->B.sizes[i] || (int64_t)p->DB.strides[i] < 0) return FA_ERROR_INVALID_VALUE;

@@ -489,6 +489,75 @@ def test_padded_and_strided_varlen(layout, causal, backend):
     _run_layout_case(layout, causal, backend, [70, 5, 192, 133], [3, 11, 0, 60], 128, torch.bfloat16, 4, 2)
 
 
+@pytest.mark.parametrize('layout', ['padded', 'compact'])
+@pytest.mark.parametrize('dtype,D', [(torch.bfloat16, 64), (torch.float16, 128), (torch.float32, 64)])
+@pytest.mark.parametrize('backend', [0, 1])
+def test_varlen_with_bias(layout, dtype, D, backend):
+    """The reference's kernels index the bias of a varlen batch by batch index and by rows and columns
+    counted from the sequence's start (modules/flash/kernel/fwd_kernel.py:393-395): one (Hq, max, max)
+    slab per sequence in the padded layout (dB likewise), one slab shared by all sequences of packed
+    tokens (no dB then).  Against the oracle, sequence by sequence."""
+    from aotriton_amd import flash
+    from oracle import fa_ref
+    if dtype == torch.float32 and backend == 1:
+        pytest.skip('fp32 has the split backend only')
+    lens = np.asarray([70, 5, 0, 131, 64])
+    n, mx, Hq, Hk = len(lens), int(lens.max()), 4, 2
+    g = torch.Generator().manual_seed(21)
+    rn = lambda *s, scale=1.0: (torch.randn(*s, generator=g) * scale).to(dtype).to(DEV)
+    cu = torch.tensor([0] + np.cumsum(lens).tolist(), dtype=torch.int32, device=DEV)
+    padded = layout == 'padded'
+    if padded:
+        q, k, v, do = rn(n, Hq, mx, D), rn(n, Hk, mx, D), rn(n, Hk, mx, D), rn(n, Hq, mx, D)
+        L = torch.zeros(n * Hq, mx, device=DEV, dtype=torch.float32)
+        sl = lambda t, i: t[i:i + 1, :, :lens[i]]
+        b = rn(n, Hq, mx, (mx + 7) // 8 * 8, scale=0.5)[..., :mx]
+        db = torch.full_like(b, float('nan'))
+    else:
+        T = int(lens.sum())
+        starts = cu.tolist()
+        q, k, v, do = rn(1, Hq, T, D), rn(1, Hk, T, D), rn(1, Hk, T, D), rn(1, Hq, T, D)
+        L = torch.zeros(Hq, T, device=DEV, dtype=torch.float32)
+        sl = lambda t, i: t[:, :, starts[i]:starts[i] + lens[i]]
+        b = rn(1, Hq, mx, (mx + 7) // 8 * 8, scale=0.5)[..., :mx]
+        db = None
+    o, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    delta = torch.zeros_like(L)
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+    sm = 1.0 / math.sqrt(D)
+    ok = flash.hipError_t.hipSuccess
+    causal = True
+    assert flash.attn_fwd_varlen(q, k, v, cu, cu, mx, mx, None, None, b, sm, L, o, 0.0, null, null, 0, null, null,
+                                 None, causal, atomic, layout) == ok
+    ext = flash.attn_options(); ext.force_backend_index = backend
+    assert flash.attn_bwd_varlen(q, k, v, cu, cu, mx, mx, None, None, b, sm, o, do, dq, dk, dv, db, None, L, delta,
+                                 0.0, null, null, 0, causal, layout, extargs=ext) == ok
+    torch.cuda.synchronize()
+    if not padded:      # a dB of packed tokens has no owner
+        assert flash.attn_bwd_varlen(q, k, v, cu, cu, mx, mx, None, None, b, sm, o, do, dq, dk, dv, torch.empty_like(b),
+                                     None, L, delta, 0.0, null, null, 0, causal, layout,
+                                     extargs=ext) == flash.hipError_t.hipErrorNotSupported
+    ct, wl, wr = flash.translate_causal(causal)
+    hp = torch.float64 if dtype == torch.float32 else torch.float32
+    f = lambda t: t.to(hp)
+    for i in range(n):
+        if lens[i] == 0:
+            continue
+        qi, ki, vi, doi = sl(q, i), sl(k, i), sl(v, i), sl(do, i)
+        bi = b[i:i + 1, :, :lens[i], :lens[i]] if padded else b[:, :, :lens[i], :lens[i]]
+        ro, rl, _ = fa_ref.attn_fwd_ref(f(qi), f(ki), f(vi), f(bi), sm, ct, wl, wr, 0.0, None)
+        lo, ll, _ = fa_ref.attn_fwd_ref(qi, ki, vi, bi, sm, ct, wl, wr, 0.0, None)
+        check(f'out[{i}]', sl(o, i), ro, lo, FUDGE['out'])
+        rg = fa_ref.attn_bwd_ref(f(qi), f(ki), f(vi), f(bi), sm, ro, f(doi), rl, ct, wl, wr, 0.0, None)
+        lg = fa_ref.attn_bwd_ref(qi, ki, vi, bi, sm, lo, doi, ll.to(dtype).float().to(dtype), ct, wl, wr, 0.0, None)
+        check(f'dq[{i}]', sl(dq, i), rg[0], lg[0], FUDGE['dq'])
+        check(f'dk[{i}]', sl(dk, i), rg[1], lg[1], FUDGE['dk'])
+        check(f'dv[{i}]', sl(dv, i), rg[2], lg[2], FUDGE['dv'])
+        if padded:
+            check(f'db[{i}]', db[i:i + 1, :, :lens[i], :lens[i]], rg[3], lg[3], FUDGE['db'])
+
+
 def _sampled_layout_cases(n=24, seed=77):
     import random
     rnd = random.Random(seed)
