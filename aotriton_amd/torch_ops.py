@@ -140,7 +140,7 @@ flash_attention_forward.register_autograd(_backward, setup_context=_setup_contex
 def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False,
                                  scale=None, enable_gqa=False):
     """torch.nn.functional.scaled_dot_product_attention on the custom ops above: 4-D fp16/bf16
-    CUDA tensors (B, H, L, E), head dims multiples of 8 up to 512.  A boolean mask becomes an
+    CUDA tensors (B, H, L, E), head dims up to 512 (multiples of 8 for the MFMA kernels).  A boolean mask becomes an
     additive one (0 / -inf); a query row that the mask hides completely yields zeros instead
     of NaN; dropout draws seed and offset from torch's CUDA generator (so torch.manual_seed
     governs it) but uses the operators' Philox stream, not the one of torch's own kernels.
@@ -175,7 +175,9 @@ def _routable(query, key, value, attn_mask, dropout_p):
     if not (key.dtype == query.dtype and value.dtype == query.dtype):
         return False
     dqk, dv = query.shape[-1], value.shape[-1]
-    if dqk > 512 or dv > 512 or key.shape[-1] != dqk:
+    # (head dims that are no multiple of 8 would run on the element-wise kernels: correct but slow, so the
+    # router leaves them to torch; scaled_dot_product_attention above takes them when called directly)
+    if dqk % 8 or dv % 8 or dqk > 512 or dv > 512 or key.shape[-1] != dqk:
         return False
     if query.shape[1] % max(key.shape[1], 1) or key.shape[1] != value.shape[1]:
         return False
