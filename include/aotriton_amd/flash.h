@@ -210,12 +210,22 @@ typedef struct fa_kernel_config {
 FA_API int fa_check_gpu(void* hip_stream);
 
 /* v3::flash::attn_fwd -- include/aotriton/flash.h:132-136,
- * modules/flash/csrc/attn_fwd.cc:48-149. */
+ * modules/flash/csrc/attn_fwd.cc:48-149.
+ * Head dims 1..512 (Dqk of Q and K, Dv of V and Out may differ), rounded up to a built one with the
+ * excess columns masked (attn_fwd.cc:76-82).  Tensors whose rows are made of aligned 16-byte pieces
+ * (head dims and strides multiples of 8 elements, 16-byte aligned bases) run on the MFMA kernels,
+ * anything else on element-wise vector-ALU kernels (same results, a few TFLOP/s).  A bias is
+ * (batch of Q, Hq, Max_seqlen_q, Max_seqlen_k); with cu_seqlens its batch index is the sequence for
+ * the padded layout and 0 for packed tokens, rows and columns count from the sequence's start
+ * (modules/flash/kernel/fwd_kernel.py:393-395). */
 FA_API int fa_attn_fwd(const fa_fwd_params* params, int32_t params_version,
                        void* hip_stream, const fa_options* options);
 
 /* v3::flash::attn_bwd -- include/aotriton/flash.h:176-180,
- * modules/flash/csrc/attn_bwd.cc:55-160. */
+ * modules/flash/csrc/attn_bwd.cc:55-160.
+ * Same tensors as the forward.  fp32 tensors, head dims above 256 and the element-wise kernels have
+ * the split backend only.  DB with packed tokens is rejected (FA_ERROR_NOT_SUPPORTED): all sequences
+ * share one bias there. */
 FA_API int fa_attn_bwd(const fa_bwd_params* params, int32_t params_version,
                        void* hip_stream, const fa_options* options);
 
