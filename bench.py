@@ -14,7 +14,7 @@ larger than the last-level cache is zeroed before every launch, warm-up >= 25 ms
 >= 100 ms of timed launches, HIP events on the launch stream, median with the 20th and
 80th percentile.  `roofline` describes the kernel that takes the largest share of the
 step; `cpu_baseline` is PyTorch's math SDPA (the reference's own test oracle) on the host
-CPU on a bounded sample of the same workload.  `c4` and `c5` time BASELINE.json's
+CPU on a bounded sample of the same workload.  `c4` and `c5` time the benchmark's
 configurations 4 (GQA, 16 packed sequences) and 5 (D=256, window + bias + dropout) at
 full size; they are extra keys, `value` stays the headline.
 """

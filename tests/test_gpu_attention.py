@@ -105,7 +105,7 @@ def test_bias_rows_without_vector_alignment(backend):
 
 
 def test_window_bias_dropout_small_config5():
-    # BASELINE config 5 at a size the oracle handles: window (left, 0) + bias + dropout 0.1
+    # the D = 256 benchmark configuration at a size the oracle handles: window (left, 0) + bias + dropout 0.1
     _run_case(1, 2, 2, 384, 384, 256, torch.float16, (100, 0), dropout_p=0.1, bias=True)
 
 

@@ -1,6 +1,6 @@
 """GPU parity tests for the packed-sequence (compact varlen) path, the dropout
 mask (bit-exact against the Philox closed form), the reference's known-answer
-tests, and size-independent properties at the BASELINE sizes."""
+tests, and size-independent properties at the full benchmark sizes."""
 import math
 
 import numpy as np
@@ -299,7 +299,7 @@ def test_per_head_counter_term_wraps_in_int32():
 
 
 def test_config5_mask_first_words_and_popcount():
-    """BASELINE config 5 mask (seed 0x1234, offset 0, p=0.1, 8192x8192) on sampled
+    """Mask of the benchmark configuration with dropout (seed 0x1234, offset 0, p=0.1, 8192x8192) on sampled
     (b, h) slices: bit-exact rows against the oracle and a keep-rate check."""
     from aotriton_amd import flash
     from oracle import philox

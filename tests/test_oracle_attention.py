@@ -22,7 +22,7 @@ def _inputs(B, Hq, Hk, Sq, Sk, D, dtype=torch.float64, seed=0, bias=False):
 
 CASES = [
     # B Hq Hk Sq Sk D causal_type wl wr bias dropout
-    (2, 4, 4, 128, 128, 64, 0, 0, 0, False, 0.0),       # BASELINE config 1
+    (2, 4, 4, 128, 128, 64, 0, 0, 0, False, 0.0),       # the benchmark configuration that runs on the CPU (fp32, D = 64)
     (1, 4, 2, 37, 53, 16, 3, TOP_LEFT, TOP_LEFT, False, 0.0),
     (1, 2, 2, 40, 24, 16, 3, BOTTOM_RIGHT, BOTTOM_RIGHT, False, 0.0),
     (1, 2, 1, 33, 47, 8, 3, 5, 3, False, 0.5),
