@@ -450,12 +450,13 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         }
     }
 #pragma unroll
+    // (the operand ring runs on from the Q rows of S into the dO rows of dP: the first dO operands are
+    // requested behind the last MFMAs of S instead of in front of the first ones of dP)
     for (int k = 0; k < KS; ++k) {
-      if (k + kAhead < KS) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Qb, row_a, k + kAhead, mb);
-      }
+      for (int mb = 0; mb < MB; ++mb)
+        xa[(k + kAhead) % (kAhead + 1)][mb] = k + kAhead < KS ? swz_read_row<T, D>(Qb, row_a, k + kAhead, mb)
+                                                              : swz_read_row<T, D>(dOb, row_a, k + kAhead - KS, mb);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kreg[k], k == 0 ? zero16 : s[mb]);
@@ -507,10 +508,6 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       vl[0] = swz_read_row<T, D>(Vt, row_a, 0, wave);
       vl[1] = swz_read_row<T, D>(Vt, row_a, 1, wave);
     }
-#pragma unroll
-    for (int k = 0; k < kAhead; ++k)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(dOb, row_a, k, mb);
 
     // element E = 16*mb + i of the tile: p (kept in s, undropped) and its operand form
     const unsigned q_d = q_none ? 0x40000000u : (unsigned)(m0 + 4 * hi - q_lo);
@@ -582,12 +579,12 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(dOb, row_a, k + kAhead, mb);
+          xa[(KS + k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(dOb, row_a, k + kAhead, mb);
       }
       if (kVLds && k + 2 < KS) vl[(k + 2) % 3] = swz_read_row<T, D>(Vt, row_a, k + 2, wave);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], kVLds ? vl[k % 3] : vreg[kVLds ? 0 : k],
+        dp[mb] = Tr::mfma(xa[(KS + k) % (kAhead + 1)][mb], kVLds ? vl[k % 3] : vreg[kVLds ? 0 : k],
                           k == 0 && kDropout ? zero16 : dp[mb]);
         const int gidx = k * MB + mb;
         if constexpr (EPG1 >= 1) {
@@ -638,7 +635,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
           if (gidx + kRing - 1 < TS * DB) ta[0][(gidx + kRing - 1) % kRing] = ta_read(dOb, gidx + kRing - 1);
           dv[db] = Tr::mfma(ta[0][gidx % kRing], pb[t], dv[db]);
         } else {
-          if (t + 1 < TS) ta[(t + 1) & 1 & (kRingTa ? 0 : 1)][db] = swz_read_tr<T, D>(dOb, tr_a0, tr_a1, t + 1, db);
+          // (the last step requests the first Q^T operands of the dK phase: TS is even, they land in ta[0])
+          ta[(t + 1) & 1 & (kRingTa ? 0 : 1)][db] = t + 1 < TS ? swz_read_tr<T, D>(dOb, tr_a0, tr_a1, t + 1, db)
+                                                               : swz_read_tr<T, D>(Qb, tr_a0, tr_a1, 0, db);
           dv[db] = Tr::mfma(ta[t & 1 & (kRingTa ? 0 : 1)][db], pb[t], dv[db]);
         }
         if constexpr (EPG3 >= 1) {
@@ -660,12 +659,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       }
     }
     // ---- dK^T += Q^T dS ----------------------------------------------------------
+    static_assert(TS % 2 == 0, "the dV phase leaves the first operands of this one in ta[0]");
     if (kRingTa) {
 #pragma unroll
       for (int gi = 0; gi < kRing - 1; ++gi) ta[0][gi] = ta_read(Qb, gi);
-    } else {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) ta[0][db] = swz_read_tr<T, D>(Qb, tr_a0, tr_a1, 0, db);
     }
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
@@ -1097,12 +1094,13 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Kb, row_a, k, mb);
 #pragma unroll
+    // (the operand ring runs on from the K rows of S into the V rows of dP: the first V operands are
+    // requested behind the last MFMAs of S instead of in front of the first ones of dP)
     for (int k = 0; k < KS; ++k) {
-      if (k + kAhead < KS) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Kb, row_a, k + kAhead, mb);
-      }
+      for (int mb = 0; mb < MB; ++mb)
+        xa[(k + kAhead) % (kAhead + 1)][mb] = k + kAhead < KS ? swz_read_row<T, D>(Kb, row_a, k + kAhead, mb)
+                                                              : swz_read_row<T, D>(Vb, row_a, k + kAhead - KS, mb);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         s[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], qreg[k], k == 0 ? zero16 : s[mb]);
@@ -1121,10 +1119,6 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int k = 0; k < kAhead; ++k)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[k][mb] = swz_read_row<T, D>(Vb, row_a, k, mb);
     if (kBias && tile_co) {
       // (the wave's LDS operations run in order: the previous tile's dB pieces have left the area)
 #pragma unroll
@@ -1194,11 +1188,11 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
       if (k + kAhead < KS) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xa[(k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Vb, row_a, k + kAhead, mb);
+          xa[(KS + k + kAhead) % (kAhead + 1)][mb] = swz_read_row<T, D>(Vb, row_a, k + kAhead, mb);
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        dp[mb] = Tr::mfma(xa[k % (kAhead + 1)][mb], doreg[k], k == 0 ? (kFoldDelta ? negd16 : zero16) : dp[mb]);
+        dp[mb] = Tr::mfma(xa[(KS + k) % (kAhead + 1)][mb], doreg[k], k == 0 ? (kFoldDelta ? negd16 : zero16) : dp[mb]);
 #pragma unroll
         for (int e = 0; e < EPG1; ++e) p_el((k * MB + mb) * EPG1 + e);
         __builtin_amdgcn_sched_barrier(0);
