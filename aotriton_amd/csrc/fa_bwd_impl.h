@@ -1319,7 +1319,7 @@ void bwd_dkdv_kernel(const BwdArgs a) {
   LevelWalk walk;
   if (ragged)
     walk.init<NW * 64>(reinterpret_cast<uint32_t*>(smem_raw + DkDvSmem<D, BM>::BYTES), a.seq, zh_lo,
-                       zh_lo + a.zh_per_xcd < a.num_zh ? zh_lo + a.zh_per_xcd : a.num_zh, a.num_zh / a.hk, NW * 32, true,
+                       zh_lo + a.zh_per_xcd < a.num_zh ? zh_lo + a.zh_per_xcd : a.num_zh, a.num_zh / a.hk, 1, NW * 32, true,
                        threadIdx.x);
   // (D = 256 is launched with one workgroup per item: the loop would cost registers there)
   for (int r = 0; D >= 256 ? r < 1 : r * workers < a.items_per_xcd; ++r) {

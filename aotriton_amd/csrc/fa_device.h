@@ -342,15 +342,18 @@ constexpr int kLevelBytes = 2 * kLevelCap * 4;
 struct LevelWalk {
   const uint32_t* tab;             // (tiles << 16 | 0xffff - entry), descending
   int count, w, base, c;           // entries; current level, position of its first item, entries that reach it
+  bool keys;                       // tiles count keys and a level is the distance to the END (dK/dV); else queries, from the start
   __device__ __forceinline__ int tiles_at(int i) const { return (int)(__builtin_amdgcn_readfirstlane(tab[i]) >> 16); }
-  // all threads of the workgroup (NT of them) call this; entries are the heads lo .. hi-1
+  // all threads of the workgroup (NT of them) call this; entries are the heads lo .. hi-1, `ratio` of
+  // them per (sequence, kv-head)
   template <int NT>
-  __device__ __forceinline__ void init(uint32_t* lds, const SeqArgs& seq, int lo, int hi, int nseq, int rows_per_tile,
-                                       bool keys, int tid) {
+  __device__ __forceinline__ void init(uint32_t* lds, const SeqArgs& seq, int lo, int hi, int nseq, int ratio,
+                                       int rows_per_tile, bool keys_, int tid) {
     count = hi - lo;
+    keys = keys_;
     uint32_t* raw = lds + kLevelCap;
     for (int i = tid; i < count; i += NT) {
-      const SeqInfo si = get_seq(seq, (lo + i) % nseq);
+      const SeqInfo si = get_seq(seq, ((lo + i) / ratio) % nseq);
       const int n = ((keys ? si.seqlen_k : si.seqlen_q) + rows_per_tile - 1) / rows_per_tile;
       raw[i] = (uint32_t)n << 16 | (uint32_t)(0xffff - i);
     }
@@ -378,7 +381,7 @@ struct LevelWalk {
     if (w <= 0) return false;
     const uint32_t key = __builtin_amdgcn_readfirstlane(tab[t - base]);
     entry = 0xffff - (int)(key & 0xffffu);
-    tile = (int)(key >> 16) - w;
+    tile = keys ? (int)(key >> 16) - w : w - 1;
     return true;
   }
 };

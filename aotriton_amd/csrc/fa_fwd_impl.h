@@ -578,16 +578,31 @@ void fwd_kernel(const FwdArgs a) {
   const int workers = gridDim.x / kNumXcd;
   const int per_group = a.zh_group * a.num_m_tiles;
   const int items = a.items_per_xcd;
-  // sequences of different lengths: the list of the valid tiles only (RaggedWalk), a set's tiles
-  // from the last one down; taken in the same serpentine order
+  // Sequences of different lengths: the list of the valid tiles only, either all tiles of the XCD's
+  // heads by their distance from the start of the sequence, the heaviest first under a causal mask
+  // (LevelWalk, up to kLevelCap heads per XCD), or set by set (RaggedWalk); taken in the same
+  // serpentine order.
   const bool ragged = a.seq.num_seqlens != 0;
   const int ratio = a.hq / a.hk, nseq = a.num_zh / a.hq;
+  const bool levels = ragged && a.zh_per_xcd <= kLevelCap && a.num_m_tiles <= 0xffff;
+  constexpr int kRows = NW * 32 * (QB > 0 ? QB : 1);
+  constexpr int kSmem = QB > 0 ? FwdPipeSmem<D, BN, (QB > 0 ? QB : 1)>::BYTES : FwdSmem<D, BN, NW>::BYTES;
+  const int zh_lo = xcd * a.zh_per_xcd;
   RaggedWalk walk;
-  if (ragged) walk.init(a.seq, xcd, a.zh_per_xcd, a.num_zh, ratio, nseq, NW * 32 * (QB > 0 ? QB : 1), false);
+  LevelWalk lwalk;
+  if (levels)
+    lwalk.init<NW * 64>(reinterpret_cast<uint32_t*>(smem_raw + kSmem), a.seq, zh_lo,
+                        zh_lo + a.zh_per_xcd < a.num_zh ? zh_lo + a.zh_per_xcd : a.num_zh, nseq, ratio, kRows, false,
+                        threadIdx.x);
+  else if (ragged) walk.init(a.seq, xcd, a.zh_per_xcd, a.num_zh, ratio, nseq, kRows, false);
   for (int r = 0;; ++r) {
     const int t = r * workers + ((r & 1) ? workers - 1 - p : p);
     int z, h, mt;
-    if (ragged) {
+    if (levels) {
+      int e;
+      if (!lwalk.at(t, e, mt)) break;
+      split_zh(zh_lo + e, nseq, ratio, z, h);
+    } else if (ragged) {
       int zh, tile;
       if (!walk.at(a.seq, t, zh, tile)) break;
       split_zh(zh, nseq, ratio, z, h);
@@ -616,7 +631,9 @@ void fwd_kernel(const FwdArgs a) {
 template <int D_, int NW_, int BN_, int QB_> struct FwdTileOf {
   static constexpr int NW = NW_, BN = BN_, QB = QB_;
   static constexpr int BM = NW * 32 * (QB > 0 ? QB : 1);
-  static constexpr int LDS = QB > 0 ? FwdPipeSmem<D_, BN, (QB > 0 ? QB : 1)>::BYTES : FwdSmem<D_, BN, NW>::BYTES;
+  // (the level table of packed sequences sits behind the item's LDS)
+  static constexpr int ITEM_LDS = QB > 0 ? FwdPipeSmem<D_, BN, (QB > 0 ? QB : 1)>::BYTES : FwdSmem<D_, BN, NW>::BYTES;
+  static constexpr int LDS = ITEM_LDS + kLevelBytes;
 };
 template <typename T, int D, bool kWindowed> struct FwdTile;
 // D = 64: 128-key tiles; 64-key tiles lose 2 % causal and 6 % non-causal at S = 4096.
