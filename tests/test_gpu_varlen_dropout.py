@@ -558,6 +558,48 @@ def test_varlen_with_bias(layout, dtype, D, backend):
             check(f'db[{i}]', db[i:i + 1, :, :lens[i], :lens[i]], rg[3], lg[3], FUDGE['db'])
 
 
+def test_packed_sequences_at_full_size_equal_per_sequence_runs():
+    """16 packed sequences of 256-8192 tokens (GQA 32 / 8, D = 128, bf16, causal: the packed benchmark
+    configuration at full size): every sequence's O, LSE, dQ, dK, dV must equal, bit for bit, what the
+    dense entry points give for that sequence alone.  The work lists of the packed run (valid tiles of
+    all sequences ordered by weight) change the order in which tiles are computed, never a result."""
+    from aotriton_amd import flash
+    ok = flash.hipError_t.hipSuccess
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    rng = np.random.default_rng(1234)
+    lens = rng.integers(256, 8193, size=16)
+    cu = np.zeros(17, dtype=np.int32)
+    cu[1:] = np.cumsum(lens)
+    T, Hq, Hk, D = int(cu[-1]), 32, 8, 128
+    gg = torch.Generator(device=DEV).manual_seed(1)
+    mk = lambda h: torch.randn(1, T, h, D, device=DEV, dtype=torch.float32, generator=gg).to(torch.bfloat16).transpose(1, 2)
+    q, k, v, do = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+    o, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    L = torch.empty(Hq, T, device=DEV, dtype=torch.float32)
+    d = torch.empty_like(L)
+    cuq = torch.from_numpy(cu).to(DEV)
+    mx, sm = int(lens.max()), 1.0 / math.sqrt(D)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+    assert flash.attn_fwd_compact_varlen(q, k, v, None, cuq, cuq, mx, mx, sm, L, o, 0.0, null, null, 0, null, null, None,
+                                         True, atomic) == ok
+    assert flash.attn_bwd_compact_varlen(q, k, v, cuq, cuq, mx, mx, None, sm, o, do, dq, dk, dv, None, L, d, 0.0, null,
+                                         null, 0, True) == ok
+    torch.cuda.synchronize()
+    for i in range(len(lens)):
+        s, n = slice(int(cu[i]), int(cu[i + 1])), int(lens[i])
+        qi, ki, vi, doi = [t[:, :, s].contiguous() for t in (q, k, v, do)]
+        oi, dqi, dki, dvi = torch.empty_like(qi), torch.empty_like(qi), torch.empty_like(ki), torch.empty_like(vi)
+        Li = torch.empty(Hq, n, device=DEV, dtype=torch.float32)
+        di = torch.empty_like(Li)
+        assert flash.attn_fwd(qi, ki, vi, None, sm, Li, oi, 0.0, null, null, 0, null, null, None, True, atomic) == ok
+        assert flash.attn_bwd(qi, ki, vi, None, sm, oi, doi, dqi, dki, dvi, None, None, Li, di, 0.0, null, null, 0,
+                              True) == ok
+        torch.cuda.synchronize()
+        for name, a, b in (('o', o[:, :, s], oi), ('lse', L[:, s], Li), ('dq', dq[:, :, s], dqi),
+                           ('dk', dk[:, :, s], dki), ('dv', dv[:, :, s], dvi)):
+            assert torch.equal(a, b), f'sequence {i}: {name} differs from the run of the sequence alone'
+
+
 def _sampled_layout_cases(n=24, seed=77):
     import random
     rnd = random.Random(seed)
