@@ -103,8 +103,9 @@ def scan(jobs=8):
     a loop exits to, before exec is restored: the store runs with no lane enabled and the reload
     later returns whatever the slot held.  The kernels here are written so that none is emitted;
     returns the list of (file, loops, functions left out of line) that have some of either."""
-    tmp = os.path.join(OBJ, 'scan')
-    os.makedirs(tmp, exist_ok=True)
+    import tempfile
+    tmpdir = tempfile.TemporaryDirectory(prefix='fa_scan_')
+    tmp = tmpdir.name
 
     def one(unit):
         src, defines, objname = unit
@@ -122,7 +123,7 @@ def scan(jobs=8):
         outlined = len(re.findall(r'^\s*\.type\s+\S+,@function', text, re.M)) - text.count('.amdhsa_kernel ')
         return objname, len(_WATERFALL.findall(text)), outlined
 
-    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+    with tmpdir, concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         return [(n, c, o) for n, c, o in ex.map(one, sources()) if c or o]
 
 
