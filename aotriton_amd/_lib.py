@@ -118,6 +118,8 @@ SYMBOLS = {
                                                              P(fa_tensor0), P(fa_tensor0), ctypes.c_int64,
                                                              ctypes.c_int32, ctypes.c_void_p]),
     'fa_attn_bwd_noalloc': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p]),
+    'fa_set_bwd_workspace_limit': (None, [ctypes.c_int64]),
+    'fa_trim_workspace': (ctypes.c_int, []),
     'fa_attn_bwd_kernel': (ctypes.c_int, [P(fa_bwd_params), ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32]),
     'fa_debug_simulate_encoded_softmax': (ctypes.c_int, [P(fa_tensor4), ctypes.c_float, P(fa_tensor0),
                                                          P(fa_tensor0), ctypes.c_uint64, ctypes.c_void_p]),

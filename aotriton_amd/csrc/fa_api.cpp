@@ -101,6 +101,85 @@ hipError_t scratch_of_device(int dev, float** out) {
   return hipSuccess;
 }
 
+// Workspace of the backward that keeps dS in HBM between its two kernels: one buffer per device
+// that belongs to the library and only grows (hipMalloc once, then reused: a stream-ordered pool
+// allocation made the host wait for the GPU on every call).  Calls on one device share it: the
+// mutex covers the enqueue, and a call on another stream than the last one first waits (on the
+// GPU) for the event recorded behind the last use.  fa_trim_workspace frees the buffers.
+std::atomic<int64_t> g_ws_limit{-1};        // bytes; -1: not set (environment, then default)
+struct Workspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  hipEvent_t done = nullptr;
+  hipStream_t last = nullptr;
+  bool used = false;
+};
+Workspace g_ws[kMaxDevices];
+std::mutex g_ws_mutex;
+
+int64_t ws_limit_bytes(int dev) {
+  int64_t v = g_ws_limit.load(std::memory_order_relaxed);
+  if (v >= 0) return v;
+  static const int64_t from_env = [] {
+    const char* e = std::getenv("AOTRITON_AMD_BWD_WORKSPACE_MB");
+    return e ? (int64_t)std::atoll(e) << 20 : (int64_t)-1;
+  }();
+  if (from_env >= 0) return from_env;
+  // default: an eighth of the device's memory (36 GB of 288)
+  static std::atomic<int64_t> dflt[kMaxDevices];
+  int64_t d = dflt[dev].load(std::memory_order_relaxed);
+  if (d == 0) {
+    hipDeviceProp_t prop;
+    d = hipGetDeviceProperties(&prop, dev) == hipSuccess ? (int64_t)(prop.totalGlobalMem / 8) : ((int64_t)1 << 30);
+    dflt[dev].store(d, std::memory_order_relaxed);
+  }
+  return d;
+}
+
+// Returns with g_ws_mutex held when it succeeds; ws_release drops it.
+hipError_t ws_acquire(int dev, size_t need, hipStream_t stream, void** out) {
+  g_ws_mutex.lock();
+  Workspace& w = g_ws[dev];
+  hipError_t e = hipSuccess;
+  if (w.bytes < need || w.done == nullptr) {
+    int cur = -1;
+    e = hipGetDevice(&cur);
+    if (e == hipSuccess && cur != dev) e = hipSetDevice(dev);
+    if (e == hipSuccess && w.done == nullptr) e = hipEventCreateWithFlags(&w.done, hipEventDisableTiming);
+    if (e == hipSuccess && w.bytes < need) {
+      // (hipFree waits for the device: nothing uses the old buffer any more)
+      if (w.ptr != nullptr) (void)hipFree(w.ptr);
+      w.ptr = nullptr; w.bytes = 0; w.used = false;
+      const size_t grow = need + need / 8;
+      e = hipMalloc(&w.ptr, grow);
+      if (e == hipSuccess) w.bytes = grow; else w.ptr = nullptr;
+    }
+    if (cur >= 0 && cur != dev) (void)hipSetDevice(cur);
+  }
+  if (e == hipSuccess && w.used && w.last != stream) e = hipStreamWaitEvent(stream, w.done, 0);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    g_ws_mutex.unlock();
+    return e;
+  }
+  *out = w.ptr;
+  return hipSuccess;
+}
+
+void ws_release(int dev, hipStream_t stream) {
+  Workspace& w = g_ws[dev];
+  if (hipEventRecord(w.done, stream) == hipSuccess) {
+    w.last = stream;
+    w.used = true;
+  } else {
+    // without the event the next call cannot order itself behind this one
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(stream);
+    w.used = false;
+  }
+  g_ws_mutex.unlock();
+}
+
 bool is_16bit(int dt) { return dt == FA_DTYPE_FLOAT16 || dt == FA_DTYPE_BFLOAT16; }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -682,6 +761,44 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     // out; the dK/dV kernel runs after it and reads it, so the whole backward is two launches
     // (kernel_slot 0 still launches the preprocess kernel on its own).
     const bool delta_launch = f32 || big || slow;
+    // The 16-bit kernels at head dims 72-128 can keep dS in HBM instead of recomputing S and dP in
+    // the dQ kernel (5 GEMMs instead of 7): delta first, then dK/dV writing dS, then dQ = dS K.  It
+    // takes 2 bytes per (query, key) pair of workspace; when that is above the limit, under stream
+    // capture, for packed sequences or with dB the kernels recompute.  (Measured at B4 S4096, bf16
+    // causal: head dim 128 gains, head dim 64, where a pair costs half the arithmetic and the same
+    // bytes, loses 13 %.)
+    void* ds_ws = nullptr;
+    if (kernel_slot < 0 && !own_delta && !delta_launch && s.d == 128 && s.num_seqlens == 0 && p->DB.ptr == nullptr &&
+        s.batch > 0 && s.max_sq > 0 && s.max_sk > 0) {
+      int ntq = 0, ntk = 0;
+      int64_t tile_bytes = 0;
+      fa::ds_tile_counts(dt, s.d, s.max_sq, s.max_sk, &ntq, &ntk, &tile_bytes);
+      const int64_t ds_bytes = (int64_t)s.batch * s.hq * ntq * ntk * tile_bytes;
+      const int64_t stat_bytes = (s.row_stats * 4 + 255) & ~(int64_t)255;
+      const int64_t need = ds_bytes + 2 * stat_bytes;
+      hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+      const bool capturing = hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+      if (!capturing && need <= ws_limit_bytes(device_index(dev))) {
+        if (ws_acquire(device_index(dev), (size_t)need, stream, &ds_ws) == hipSuccess) {
+          a.ds_ntq = ntq;
+          a.ds_ntk = ntk;
+          a.lse_scaled = reinterpret_cast<const float*>(static_cast<char*>(ds_ws) + ds_bytes);
+          a.delta_prep = reinterpret_cast<const float*>(static_cast<char*>(ds_ws) + ds_bytes + stat_bytes);
+        } else {
+          ds_ws = nullptr;
+          FA_LOG(2, "attn_bwd: no workspace of %lld bytes for dS, recomputing instead", (long long)need);
+        }
+      }
+    }
+    if (ds_ws != nullptr) {
+      err = fa::run_bwd_preprocess(dt, s.d, a, stream);
+      a.ds_ws = ds_ws;
+      if (err == hipSuccess) err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      if (err == hipSuccess) err = fa::run_bwd_dqs(dt, s.d, a, stream);
+      ws_release(device_index(dev), stream);
+      if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);
+      return (int)err;
+    }
     if (kernel_slot == 0 || (kernel_slot < 0 && delta_launch))
       err = delta_launch ? fa::run_bwd_valu(dt, s.d, 0, a, stream) : fa::run_bwd_preprocess(dt, s.d, a, stream);
     const int order[2] = {delta_launch ? 1 : 2, delta_launch ? 2 : 1};
@@ -837,6 +954,20 @@ int fa_v2_attn_bwd_compact_varlen(const fa_tensor4* q, const fa_tensor4* k, cons
   return v2_bwd(q, k, v, b, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, sm_scale, out, dout, dq, dk,
                 dv, db, softmax_lse, delta, dropout_p, philox_seed, philox_offset1, philox_offset2, is_causal, 0,
                 hip_stream);
+}
+
+void fa_set_bwd_workspace_limit(int64_t bytes) { g_ws_limit.store(bytes, std::memory_order_relaxed); }
+
+int fa_trim_workspace(void) {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  hipError_t err = hipSuccess;
+  for (int d = 0; d < kMaxDevices; ++d)
+    if (g_ws[d].ptr != nullptr) {
+      const hipError_t e = hipFree(g_ws[d].ptr);      // waits for the device first
+      g_ws[d].ptr = nullptr; g_ws[d].bytes = 0; g_ws[d].used = false;
+      if (err == hipSuccess) err = e;
+    }
+  return (int)err;
 }
 
 int fa_attn_bwd_noalloc(const fa_bwd_params* p, int32_t params_version, void* hip_stream) {

@@ -79,6 +79,13 @@ struct BwdArgs {
   int32_t zh_group;      // heads walked together on one XCD
   int32_t num_cu;        // CUs of the device (host fills it in)
   int32_t items_per_xcd; // work items (incl. padding of the last group) per XCD
+  // dS kept in HBM between the dK/dV kernel (writes it) and the dQ kernel that only does dQ = dS K:
+  // tiles of 128 keys x (the dK/dV step's queries), ds_ntk x ds_ntq of them per (batch element, q-head)
+  void* ds_ws;           // null: dS is not stored
+  int32_t ds_ntq, ds_ntk;
+  // with ds_ws: row statistics as that dK/dV kernel stages them, written by the delta kernel
+  const float* lse_scaled;   // L / ln 2
+  const float* delta_prep;   // -delta (delta with dropout)
 };
 
 struct EncodedSoftmaxArgs {

@@ -29,7 +29,10 @@ namespace fa {
 // ---------------------------------------------------------------------------
 // delta = rowsum(O * dO) in fp32, same layout as LSE.
 // ---------------------------------------------------------------------------
-template <typename T, int D>
+// kPrep: also writes what the dK/dV kernel that stores dS stages without touching it: L in base 2
+// (BwdArgs::lse_scaled) and the initial value of its dP accumulators (delta_prep: -delta, or delta
+// itself when dropout comes between dP and the subtraction).
+template <typename T, int D, bool kPrep = false>
 __global__ void bwd_preprocess_kernel(const BwdArgs a) {
   using op_t = typename Traits<T>::op_t;
   constexpr int LPR = D / 8;               // lanes per row
@@ -50,7 +53,14 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
   }
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (row < si.seqlen_q && cc == 0) a.delta[lse_offset(si, h, a.hq) + row] = acc;
+  if (row < si.seqlen_q && cc == 0) {
+    const int64_t at = lse_offset(si, h, a.hq) + row;
+    a.delta[at] = acc;
+    if constexpr (kPrep) {
+      const_cast<float*>(a.lse_scaled)[at] = a.lse[at] * kRcpLn2;          // bwd_inner_dk_dv.py:185-186
+      const_cast<float*>(a.delta_prep)[at] = a.drop.p > 0.f ? acc : -acc;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -95,10 +105,31 @@ template <typename T, bool kWindowed> struct BwdTile<T, 64, kWindowed>  { static
 template <typename T, bool kWindowed> struct BwdTile<T, 128, kWindowed> { static constexpr int NW = 4, DKDV_BM = 64, DQ_BN = 64; };
 template <typename T, bool kWindowed> struct BwdTile<T, 256, kWindowed> { static constexpr int NW = 4, DKDV_BM = 32, DQ_BN = 32; };
 
+// Stored dS (BwdArgs::ds_ws): one tile per (batch element, q-head, key tile of 128, query tile of the
+// dK/dV step) holds 128 x BM values of the 16-bit type as [32-query block][32-key block][half of the
+// query block][64 pieces of 16 bytes].  A piece is what one lane of the dK/dV item holds as the MFMA
+// operand of its 16-query step t (query block t / 2, half t % 2): its key c (lane % 32) against the
+// queries 16 t + 4 hi + {0..3} and 16 t + 8 + 4 hi + {0..3} (hi = lane / 32); it sits at piece position
+// (2 c + hi) ^ 8 (t & 1), where the transposing LDS reads of the kernel that consumes the tiles want
+// it.  A wave of that kernel owns one query block: what it needs of a tile is contiguous.
+template <typename T, int D> struct DsTile {
+  static_assert(BwdTile<T, D, false>::DKDV_BM == BwdTile<T, D, true>::DKDV_BM, "one tile shape per head dim");
+  static constexpr int BM = BwdTile<T, D, false>::DKDV_BM;   // queries per stored tile
+  static constexpr int BN = 128;                             // keys per stored tile
+  static constexpr int TS = BM / 16;                         // 1 KB pieces per 32-key block
+  static constexpr int BYTES = BN * BM * 2;
+  static constexpr int QBLOCK_BYTES = BN * 32 * 2;           // one 32-query block against the tile's keys
+  // byte offset of the piece of 32-key block kw and 16-query step t
+  static constexpr int piece(int kw, int t) { return (t >> 1) * QBLOCK_BYTES + kw * 2048 + (t & 1) * 1024; }
+};
+
 // ---------------------------------------------------------------------------
 // dK / dV work item
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta, bool kPad>
+// kStoreDs: dS of every visited tile pair is also written to BwdArgs::ds_ws, and the row statistics
+// come prepared (BwdArgs::lse_scaled, delta_prep) so that they can travel straight into LDS.
+template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kInlineDelta, bool kPad,
+          bool kStoreDs = false>
 __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const int nt, const int z,
                                           char* smem_raw) {
   using Tr = Traits<T>;
@@ -114,6 +145,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, hi = lane >> 5;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
   // columns of Q/K/dQ/dK and of V/Out/dOut/dV: <= D, multiples of 8; constants unless a head dim is rounded up
   const int d_qk = kPad ? a.head_dim : D, d_v = kPad ? a.head_dim_v : D;
 
@@ -193,6 +225,32 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 
   auto stage_ptr = [&](int stage) { return smem_raw + stage * SM::STAGE_BYTES; };
 
+  // dS of every visited (key tile, query tile) pair goes out to HBM for the kernel that forms dQ from
+  // it: the operand registers of the dK GEMM as they are, 1 KB per wave instruction.  A store counts
+  // in vmcnt until the L2 has taken it, which takes 1700-1900 cycles for a line that misses; loads
+  // and stores complete out of order with respect to each other, so the next wait for a load is a
+  // wait for every store before it.  The tile therefore has ONE wait for vector memory, in its
+  // middle (where the compiler makes the first transposing read wait for the direct-to-LDS pieces
+  // anyway), and the pieces leave in the half tile after it, as their operands get complete: the
+  // youngest store is more than half a tile old at the next wait.
+  using DT = DsTile<T, D>;
+  static_assert(!kStoreDs || (!kInlineDelta && BM == DT::BM && BN == DT::BN), "stored tiles have the item's shape");
+  const int ds_pos[2] = {((c << 1) | hi) << 4, (((c << 1) | hi) ^ 8) << 4};
+  op_t sb[TS];                         // dS operands of the dK GEMM; with kStoreDs they outlive their tile
+  char* ds_tile = nullptr;             // stored tile of the running (q-head, Q tile) step
+  constexpr int kDsSlots = 4;
+  auto ds_slot_of = [](int t) { return TS >= kDsSlots ? t * kDsSlots / TS : 2 * t + 1; };
+  auto store_ds_slot = [&](char* tile, int slot) {
+    if constexpr (kStoreDs) {
+      const auto rs = __builtin_amdgcn_make_buffer_rsrc(tile, 0, tile != nullptr ? DT::BYTES : 0, 0x00020000);
+#pragma unroll
+      for (int t = 0; t < TS; ++t)
+        if (ds_slot_of(t) == slot)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sb[t]), rs, ds_pos[t & 1],
+                                                 DT::piece(0, t) + wave_u * 2048, 2);
+    }
+  };
+
   // ---- staging -----------------------------------------------------------------
   // Q and dO tiles travel global -> registers -> LDS in 16-byte pieces.  The pieces
   // are issued between the MFMAs of the running tile (loads behind S = Q K^T, LDS
@@ -216,7 +274,6 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   op_t qch[kDirect ? 1 : CH], doch[kDirect ? 1 : CH], och[kInlineDelta ? CH : 1];
   float l_stage = 0.f, d_stage = 0.f;
   const int r0 = tid / LPR, cc0 = tid % LPR;
-  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
   int f_stage = 0;                               // stage the running fetch fills
   // f(r0 + k RPI) takes at most two values, for even and odd k (RPI is a multiple of 8, f has period 16)
   int q_voff_d[2] = {0, 0}, do_voff_d[2] = {0, 0};
@@ -253,8 +310,8 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     if (kInlineDelta)
       ob = reinterpret_cast<const T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)hq * a.so.h +
            row0 * a.so.s;
-    lse_b = a.lse + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
-    if (!kInlineDelta) delta_b = a.delta + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
+    lse_b = (kStoreDs ? a.lse_scaled : a.lse) + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
+    if (!kInlineDelta) delta_b = (kStoreDs ? a.delta_prep : a.delta) + lse_offset(si, hq, a.hq) + (int64_t)br.lo * BM;
   };
   __amdgpu_buffer_rsrc_t q_rs, do_rs, o_rs, b_rs;
   // The bias tile (BM queries x the workgroup's 128 keys) is staged through LDS like Q
@@ -297,7 +354,18 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     if (kInlineDelta)
       o_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ob), 0,
                                                any ? ((rows - 1) * (int)a.so.s + d_v) * 2 : 0, 0x00020000);
-    if (tid < BM) {
+    if constexpr (kStoreDs) {
+      // the prepared statistics (L log2e; -delta, or delta with dropout) go straight into the stage:
+      // no register load in the loop, hence no wait of the compiler's for one at the end of a tile
+      // (16 bytes per lane: BM / 4 lanes of wave 0 fetch each array)
+      if (tid < BM / 4) {
+        const auto l_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(lse_b), 0, rows * 4, 0x00020000);
+        const auto d_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(delta_b), 0, rows * 4, 0x00020000);
+        char* st = stage_ptr(f_stage) + 2 * SM::TILE_BYTES;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(l_rs, (lds_ptr_t)st, 16, lane * 16, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(d_rs, (lds_ptr_t)(st + BM * 4), 16, lane * 16, 0, 0, 0);
+      }
+    } else if (tid < BM) {
       const bool ok = tid < rows;
       l_stage = ok ? lse_b[tid] : 0.f;
       if (!kInlineDelta) d_stage = ok ? delta_b[tid] : 0.f;
@@ -391,7 +459,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         if (cc0 == 0) Ds[r0 + k * RPI] = kDropout ? acc : -acc;
       }
     }
-    if (tid < BM) {
+    if (!kStoreDs && tid < BM) {
       Ls[tid] = l_stage * kRcpLn2;                          // bwd_inner_dk_dv.py:185-186
       // without dropout -delta is staged: it is the initial value of the dP accumulators
       if (!kInlineDelta) Ds[tid] = kDropout ? d_stage : -d_stage;
@@ -420,13 +488,19 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
 
     DropoutState dst{};
     if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
+    if constexpr (kStoreDs) {
+      // (the tiles of a q-head follow each other)
+      ds_tile = e == 0 ? reinterpret_cast<char*>(a.ds_ws) +
+                             ((((int64_t)z * a.hq + hq) * a.ds_ntk + nt) * a.ds_ntq + br.lo) * DT::BYTES
+                       : ds_tile + DT::BYTES;
+    }
 
     // The vector ALU work is spread over the MFMAs of the GEMMs that do not depend on
     // it: p = exp2(...) of S runs behind the MFMAs of dP, ds = p (dP - delta) behind
     // those of dV.  Fences keep the hand-made order.
     constexpr int kAhead = D >= 256 ? 1 : 2;
     op_t xa[kAhead + 1][MB];
-    op_t pb[TS], sb[TS];
+    op_t pb[TS];
     uint32_t kw[kDropout ? MB : 1][4];
     // row statistics are read four rows at a time, one read ahead of their use
     f32x4 l4[2], d4[2];
@@ -606,6 +680,11 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    // With stored dS this is the tile's only wait for vector memory: everything the S phase requested
+    // for the next tile has arrived (the compiler makes the first transposing read below wait for
+    // the direct-to-LDS pieces anyway), and the stores issued since the last wait are at least a
+    // phase and a half old.
+    if constexpr (kStoreDs) direct_landed();
     // delta of the tile's queries, first transposed dO operands
     if (kDropout) d4[0] = *reinterpret_cast<const f32x4*>(stat_ptr(Ds, 0));
     // Transposed operands are read ahead of their MFMAs: a whole 16-query step ahead, or,
@@ -655,9 +734,12 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
             if (E & 1) ds_pair(E);
           }
         }
+        if (kStoreDs && TS >= kDsSlots && gidx == G3 / 2) store_ds_slot(ds_tile, 0);
+        if (kStoreDs && gidx == 3 * G3 / 4) store_ds_slot(ds_tile, 1);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    if constexpr (kStoreDs && TS >= kDsSlots) store_ds_slot(ds_tile, 2);
     // ---- dK^T += Q^T dS ----------------------------------------------------------
     static_assert(TS % 2 == 0, "the dV phase leaves the first operands of this one in ta[0]");
     if (kRingTa) {
@@ -680,6 +762,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         } else {
           dk[db] = Tr::mfma(ta[t & 1 & (kRingTa ? 0 : 1)][db], sb[t], dk[db]);
         }
+        if (kStoreDs && t * DB + db == 2) store_ds_slot(ds_tile, 3);
         // the next tile's LDS writes ride behind these MFMAs
         constexpr int per = (STORE_PIECES + G4 - 1) / G4;
 #pragma unroll
@@ -691,7 +774,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       __builtin_amdgcn_sched_barrier(0);
     }
     store_stats(stage ^ 1);
-    direct_landed();
+    if constexpr (!kStoreDs) direct_landed();
   };
 
   if (kVLds) {
@@ -1300,7 +1383,7 @@ __host__ __device__ inline bool dkdv_level_list(const BwdArgs& a) {
   return D < 256 && a.seq.num_seqlens != 0 && a.bias == nullptr && a.zh_per_xcd <= kLevelCap && a.num_n_tiles <= 0xffff;
 }
 
-template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kPad>
+template <typename T, int D, int NW, int BM, bool kWindowed, bool kBias, bool kDropout, bool kPad, bool kStoreDs = false>
 __global__ __attribute__((amdgpu_flat_work_group_size(NW * 64, NW * 64)))
 void bwd_dkdv_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -1339,7 +1422,7 @@ void bwd_dkdv_kernel(const BwdArgs a) {
     }
     int z, hk;
     split_zh(zh, a.num_zh / a.hk, 1, z, hk);
-    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad>(a, hk, nt, z, smem_raw);
+    dkdv_item<T, D, NW, BM, kWindowed, kBias, kDropout, false, kPad, kStoreDs>(a, hk, nt, z, smem_raw);
     __syncthreads();     // the next item reuses the LDS stages
   }
 }
@@ -1455,7 +1538,10 @@ hipError_t launch_bwd_preprocess(const BwdArgs& a, hipStream_t stream) {
   constexpr int ROWS = 256 / (D / 8);
   dim3 grid((a.seq.max_seqlen_q + ROWS - 1) / ROWS, a.hq, bwd_nseq(a));
   if (grid.x == 0 || grid.z == 0) return hipSuccess;
-  hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), grid, dim3(256), 0, stream, a);
+  if (a.lse_scaled != nullptr)
+    hipLaunchKernelGGL((bwd_preprocess_kernel<T, D, true>), grid, dim3(256), 0, stream, a);
+  else
+    hipLaunchKernelGGL((bwd_preprocess_kernel<T, D, false>), grid, dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 
@@ -1472,6 +1558,13 @@ hipError_t launch_dkdv_variant(const BwdArgs& a0, hipStream_t stream) {
   dim3 grid((unsigned)(kNumXcd * persistent_workers<D>(a)));
   // (the level table's LDS is requested whether or not this launch uses it: the kernel's limit is set once)
   constexpr int smem = DkDvSmem<D, BM>::BYTES + (D < 256 ? kLevelBytes : 0);
+  if (a.ds_ws != nullptr) {
+    // (the variant that stores dS exists where it pays: the 128-column build)
+    if constexpr (D == 128)
+      return launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad, true>>(grid, NW * 64, smem, stream, a);
+    else
+      return hipErrorNotSupported;
+  }
   return launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad>>(grid, NW * 64, smem, stream, a);
 }
 

@@ -30,6 +30,9 @@ hipError_t run_bwd_dkdv(int dtype, int head_dim, const BwdArgs& a, bool windowed
 hipError_t run_bwd_dq(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 hipError_t run_bwd_fused(int dtype, int head_dim, const BwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s);
 TileShape bwd_tile_shape(int dtype, int head_dim, bool windowed, int kernel_slot);
+// dQ = dS K from the dS tiles that the dK/dV kernel stored (BwdArgs::ds_ws), and their geometry
+hipError_t run_bwd_dqs(int dtype, int head_dim, const BwdArgs& a, hipStream_t s);
+void ds_tile_counts(int dtype, int head_dim, int max_sq, int max_sk, int* ntq, int* ntk, int64_t* tile_bytes);
 
 // MFMA kernels of the 16-bit types for head dims above 256, rounded up to 512 (the head dim split
 // over the waves of a workgroup).  kernel_slot of the backward: 1 dK/dV, 2 dQ and dB.

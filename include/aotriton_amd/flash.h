@@ -286,6 +286,21 @@ FA_API int fa_v2_attn_bwd_compact_varlen(
 FA_API int fa_attn_bwd_noalloc(const fa_bwd_params* params, int32_t params_version,
                                void* hip_stream);
 
+/* Workspace of the split backward.  For 16-bit tensors at head dims 72-128 (dense batches, no dB,
+ * not under stream capture) fa_attn_bwd keeps dS in HBM between its dK/dV and dQ kernels instead of
+ * recomputing S and dP in the dQ kernel (5 GEMMs instead of 7; delta kernel, dK/dV kernel writing dS,
+ * dQ = dS K kernel): 2 bytes per (batch, q-head, query, key) plus 8 bytes per (batch, q-head, query),
+ * in a buffer per device that belongs to the library, is allocated on first use, only grows and is
+ * reused by every later call (calls on one device take turns: a call on another stream than the last
+ * one waits on the GPU for the last one's kernels).  A call that would need more than the limit
+ * recomputes instead, with the same results up to fp32 summation order.  The limit is, in this
+ * order: the last fa_set_bwd_workspace_limit(bytes >= 0); AOTRITON_AMD_BWD_WORKSPACE_MB of the
+ * environment; an eighth of the device's memory.  0 switches the workspace off.  fa_trim_workspace
+ * waits for the devices and frees the buffers.  Neither has a counterpart in the reference, whose
+ * split backward always recomputes (modules/flash/kernel/bwd_kernel_dq.py:45-389). */
+FA_API void fa_set_bwd_workspace_limit(int64_t bytes);
+FA_API int fa_trim_workspace(void);
+
 /* One kernel of the backward only: kernel_slot 0 = delta (bwd_preprocess), 1 = dK/dV
  * (reads delta), 2 = dQ (16-bit types up to head dim 256: computes delta and writes it;
  * otherwise reads it), 3 = fused.  Slots 0-2 need an eager delta buffer in params->D.  Stands in
