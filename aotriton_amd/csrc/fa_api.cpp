@@ -433,6 +433,21 @@ fa::DropoutArgs dropout_args(float p, const fa_tensor0& seed, const fa_tensor0& 
   return d;
 }
 
+// Bytes of workspace with which the split backward keeps dS in HBM, 0 when this call recomputes S
+// and dP in its dQ kernel instead (anything but the 16-bit MFMA kernels of the 128-column build,
+// packed sequences, dB wanted, an empty tensor).  *ds_bytes / *stat_bytes: the parts of the buffer.
+int64_t ds_workspace_need(const fa_bwd_params* p, const Shape& s, int* ntq, int* ntk, int64_t* ds_bytes,
+                          int64_t* stat_bytes) {
+  if (s.elementwise || !is_16bit(p->Q.dtype) || s.d != 128 || s.num_seqlens != 0 || p->DB.ptr != nullptr ||
+      s.batch <= 0 || s.max_sq <= 0 || s.max_sk <= 0)
+    return 0;
+  int64_t tile_bytes = 0;
+  fa::ds_tile_counts(p->Q.dtype, s.d, s.max_sq, s.max_sk, ntq, ntk, &tile_bytes);
+  *ds_bytes = (int64_t)s.batch * s.hq * *ntq * *ntk * tile_bytes;
+  *stat_bytes = (s.row_stats * 4 + 255) & ~(int64_t)255;
+  return *ds_bytes + 2 * *stat_bytes;
+}
+
 }  // namespace
 
 extern "C" {
@@ -591,6 +606,15 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   out->backend_index = be;
   out->head_dim = s.d;
   out->flags = (s.windowed ? 1 : 0) | (s.bias ? 2 : 0) | (s.dropout ? 4 : 0) | (s.num_seqlens != 0 ? 8 : 0);
+  // 16: fa_attn_bwd would keep dS in HBM for this call on the current device (workspace within the
+  // limit; a call under stream capture recomputes all the same)
+  if (be == 0) {
+    int ntq = 0, ntk = 0, dev = 0;
+    int64_t ds_bytes = 0, stat_bytes = 0;
+    const int64_t need = ds_workspace_need(params, s, &ntq, &ntk, &ds_bytes, &stat_bytes);
+    if (need > 0 && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices && need <= ws_limit_bytes(dev))
+      out->flags |= 16;
+  }
   return FA_SUCCESS;
 }
 
@@ -768,17 +792,13 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     // causal: head dim 128 gains, head dim 64, where a pair costs half the arithmetic and the same
     // bytes, loses 13 %.)
     void* ds_ws = nullptr;
-    if (kernel_slot < 0 && !own_delta && !delta_launch && s.d == 128 && s.num_seqlens == 0 && p->DB.ptr == nullptr &&
-        s.batch > 0 && s.max_sq > 0 && s.max_sk > 0) {
-      int ntq = 0, ntk = 0;
-      int64_t tile_bytes = 0;
-      fa::ds_tile_counts(dt, s.d, s.max_sq, s.max_sk, &ntq, &ntk, &tile_bytes);
-      const int64_t ds_bytes = (int64_t)s.batch * s.hq * ntq * ntk * tile_bytes;
-      const int64_t stat_bytes = (s.row_stats * 4 + 255) & ~(int64_t)255;
-      const int64_t need = ds_bytes + 2 * stat_bytes;
+    int ntq = 0, ntk = 0;
+    int64_t ds_bytes = 0, stat_bytes = 0;
+    const int64_t need = kernel_slot < 0 && !own_delta ? ds_workspace_need(p, s, &ntq, &ntk, &ds_bytes, &stat_bytes) : 0;
+    if (need > 0 && need <= ws_limit_bytes(device_index(dev))) {
       hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
       const bool capturing = hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
-      if (!capturing && need <= ws_limit_bytes(device_index(dev))) {
+      if (!capturing) {
         if (ws_acquire(device_index(dev), (size_t)need, stream, &ds_ws) == hipSuccess) {
           a.ds_ntq = ntq;
           a.ds_ntk = ntk;

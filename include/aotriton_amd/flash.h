@@ -202,7 +202,7 @@ typedef struct fa_kernel_config {
   int32_t grid[3];
   int32_t backend_index;
   int32_t head_dim;
-  int32_t flags; /* bit0 causal/windowed, bit1 bias, bit2 dropout, bit3 varlen */
+  int32_t flags; /* bit0 causal/windowed, bit1 bias, bit2 dropout, bit3 varlen, bit4 (backward) dS kept in HBM */
 } fa_kernel_config;
 
 /* v2::flash::check_gpu -- modules/flash/csrc/attn_check.cc:36-46.
@@ -295,7 +295,8 @@ FA_API int fa_attn_bwd_noalloc(const fa_bwd_params* params, int32_t params_versi
  * one waits on the GPU for the last one's kernels).  A call that would need more than the limit
  * recomputes instead, with the same results up to fp32 summation order.  The limit is, in this
  * order: the last fa_set_bwd_workspace_limit(bytes >= 0); AOTRITON_AMD_BWD_WORKSPACE_MB of the
- * environment; an eighth of the device's memory.  0 switches the workspace off.  fa_trim_workspace
+ * environment; an eighth of the device's memory.  0 switches the workspace off, a negative value
+ * forgets the last call.  fa_query_bwd_config sets bit 4 of `flags` when a call would use it.  fa_trim_workspace
  * waits for the devices and frees the buffers.  Neither has a counterpart in the reference, whose
  * split backward always recomputes (modules/flash/kernel/bwd_kernel_dq.py:45-389). */
 FA_API void fa_set_bwd_workspace_limit(int64_t bytes);

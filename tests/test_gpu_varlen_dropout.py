@@ -558,11 +558,13 @@ def test_varlen_with_bias(layout, dtype, D, backend):
             check(f'db[{i}]', db[i:i + 1, :, :lens[i], :lens[i]], rg[3], lg[3], FUDGE['db'])
 
 
-def test_packed_sequences_at_full_size_equal_per_sequence_runs():
+def test_packed_sequences_at_full_size_equal_per_sequence_runs(recomputing_backward):
     """16 packed sequences of 256-8192 tokens (GQA 32 / 8, D = 128, bf16, causal: the packed benchmark
     configuration at full size): every sequence's O, LSE, dQ, dK, dV must equal, bit for bit, what the
     dense entry points give for that sequence alone.  The work lists of the packed run (valid tiles of
-    all sequences ordered by weight) change the order in which tiles are computed, never a result."""
+    all sequences ordered by weight) change the order in which tiles are computed, never a result.
+    (Both sides on the recomputing kernels: packed sequences always take them, and the backward that
+    keeps dS in HBM forms delta in another kernel, i.e. in another summation order.)"""
     from aotriton_amd import flash
     ok = flash.hipError_t.hipSuccess
     null = torch.empty([0], device=DEV, dtype=torch.uint64)
