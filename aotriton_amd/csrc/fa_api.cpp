@@ -684,7 +684,7 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
 }
 
 // kernel_slot < 0: the whole backward of the chosen backend; otherwise only that
-// kernel (0 delta, 1 dK/dV, 2 dQ, 3 fused).
+// kernel (0 delta, 1 dK/dV, 2 dQ, 3 fused; 4-6 the three kernels of the backward that keeps dS).
 // own_delta: the split backend with delta in the library's own per-device array (params->D is
 // not looked at).
 static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void* hip_stream,
@@ -725,7 +725,7 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     }
   }
   if (kernel_slot >= 0) {
-    forced.force_backend_index = kernel_slot == 3 ? 1 : 0;
+    forced.force_backend_index = kernel_slot == 3 ? 1 : 0;   // (slots 4-6 belong to the split backend too)
     forced.deterministic = 0;
     options = &forced;
   }
@@ -794,7 +794,14 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     void* ds_ws = nullptr;
     int ntq = 0, ntk = 0;
     int64_t ds_bytes = 0, stat_bytes = 0;
-    const int64_t need = kernel_slot < 0 && !own_delta ? ds_workspace_need(p, s, &ntq, &ntk, &ds_bytes, &stat_bytes) : 0;
+    // (kernel_slot 4, 5, 6: one kernel of this backward only; the buffer keeps its content between calls)
+    const int ds_slot = kernel_slot >= 4 ? kernel_slot - 4 : -1;
+    const int64_t need = (kernel_slot < 0 || ds_slot >= 0) && !own_delta
+                             ? ds_workspace_need(p, s, &ntq, &ntk, &ds_bytes, &stat_bytes) : 0;
+    if (ds_slot >= 0 && (need == 0 || need > ws_limit_bytes(device_index(dev)))) {
+      if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);
+      return FA_ERROR_NOT_SUPPORTED;
+    }
     if (need > 0 && need <= ws_limit_bytes(device_index(dev))) {
       hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
       const bool capturing = hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
@@ -810,11 +817,16 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
         }
       }
     }
+    if (ds_slot >= 0 && ds_ws == nullptr) {
+      if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);
+      return FA_ERROR_NOT_SUPPORTED;          // under stream capture, or no memory
+    }
     if (ds_ws != nullptr) {
-      err = fa::run_bwd_preprocess(dt, s.d, a, stream);
+      if (ds_slot < 0 || ds_slot == 0) err = fa::run_bwd_preprocess(dt, s.d, a, stream);
       a.ds_ws = ds_ws;
-      if (err == hipSuccess) err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
-      if (err == hipSuccess) err = fa::run_bwd_dqs(dt, s.d, a, stream);
+      if (err == hipSuccess && (ds_slot < 0 || ds_slot == 1))
+        err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
+      if (err == hipSuccess && (ds_slot < 0 || ds_slot == 2)) err = fa::run_bwd_dqs(dt, s.d, a, stream);
       ws_release(device_index(dev), stream);
       if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);
       return (int)err;
@@ -996,7 +1008,7 @@ int fa_attn_bwd_noalloc(const fa_bwd_params* p, int32_t params_version, void* hi
 
 int fa_attn_bwd_kernel(const fa_bwd_params* p, int32_t params_version, void* hip_stream,
                        int32_t kernel_slot) {
-  if (kernel_slot < 0 || kernel_slot > 3) return FA_ERROR_INVALID_VALUE;
+  if (kernel_slot < 0 || kernel_slot > 6) return FA_ERROR_INVALID_VALUE;
   return attn_bwd_impl(p, params_version, hip_stream, nullptr, kernel_slot);
 }
 

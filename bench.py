@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-attention hot path on one MI355X.
 
-A step = one forward + one backward (split backend) at the headline
-configuration: B=4, Hq=Hkv=32, Sq=Sk=4096, D=128, bf16, causal, q/k/v/dO ~ N(0,1)
+A step = one forward + one backward (split backend, as fa_attn_bwd runs it by default:
+at this shape dS is kept in the library's HBM workspace between the dK/dV and the dQ
+kernel) at the headline configuration: B=4, Hq=Hkv=32, Sq=Sk=4096, D=128, bf16, causal, q/k/v/dO ~ N(0,1)
 from a seed, sm_scale = 1/sqrt(128), inputs resident in HBM.  FLOP conventions
 are the reference's (modules/flash/tests/performance_forward.py:108-113):
 forward 4*B*H*S^2*D*0.5 (causal), backward 2.5x forward.
@@ -37,7 +38,8 @@ def hbm_bytes_from_profile(kernel):
     """HBM bytes per launch of `kernel` at the headline shape: the 'total ... B' figure of the
     committed rocprofv3 summary of that kernel (FETCH_SIZE / WRITE_SIZE runs, scaled by a
     256 MiB elementwise probe).  Counters cannot be read from inside this process."""
-    names = {'fwd_kernel': 'attn_fwd', 'bwd_dkdv_kernel': 'bwd_dkdv', 'bwd_dq_kernel': 'bwd_dq'}
+    names = {'fwd_kernel': 'attn_fwd', 'bwd_dkdv_kernel': 'bwd_dkdv', 'bwd_dq_kernel': 'bwd_dq',
+             'bwd_dkdv_kernel (storing dS)': 'bwd_dkdv_storing_ds', 'bwd_dqs_kernel': 'bwd_dqs'}
     path = os.path.join(ROOT, 'profiles', f'{names.get(kernel, kernel)}_b4_h32_s4096_d128_bf16_causal.txt')
     try:
         m = re.search(r'total ([0-9.e+]+) B', open(path).read())
@@ -219,14 +221,16 @@ def main():
     sm = 1.0 / math.sqrt(D)
 
     def fwd():
-        atomic.zero_()
+        # (the persistent counter is accepted and not used: the work lists are static, nothing has to be zeroed)
         assert flash.attn_fwd(q, k, v, None, sm, L, o, 0.0, null, null, 0, null, null, None, causal, atomic) == ok
 
-    def bwd(backend):
+    def bwd(backend, workspace=True):
+        lib.fa_set_bwd_workspace_limit(-1 if workspace else 0)      # 0: the dQ kernel recomputes S and dP
         ext = flash.attn_options()
         ext.force_backend_index = backend
         assert flash.attn_bwd(q, k, v, None, sm, o, do, dq, dk, dv, None, None, L, delta, 0.0, null, null, 0,
                               causal, extargs=ext) == ok
+        lib.fa_set_bwd_workspace_limit(-1)
 
     bparams = attn_bwd_params()
     flash._fill_bwd(bparams, q, k, v, None, sm, o, do, dq, dk, dv, None, None, L, delta, 0.0, null, null, 0, causal)
@@ -255,7 +259,7 @@ def main():
     torch.cuda.synchronize()
     step_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     if args.plain:
-        for slot in (0, 1, 2, 3):
+        for slot in (0, 1, 2, 3, 4, 5, 6):
             for _ in range(3):
                 bwd_slot(slot)
         torch.cuda.synchronize()
@@ -264,10 +268,15 @@ def main():
 
     r_fwd = do_bench(fwd)
     r_split = do_bench(lambda: bwd(0))
+    r_recomp = do_bench(lambda: bwd(0, workspace=False))
     r_fused = do_bench(lambda: bwd(1))
     r_pre = do_bench(lambda: bwd_slot(0))
     r_dkdv = do_bench(lambda: bwd_slot(1))
     r_dq = do_bench(lambda: bwd_slot(2))
+    bwd(0)                                        # the workspace holds this shape's dS for slot 6
+    r_prep = do_bench(lambda: bwd_slot(4))
+    r_dkdv_s = do_bench(lambda: bwd_slot(5))
+    r_dqs = do_bench(lambda: bwd_slot(6))
     torch.cuda.synchronize()
 
     f_fwd = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
@@ -281,31 +290,33 @@ def main():
             d.update(extra)
         return d
 
-    # Dominant kernel of the step and the GEMM work it is required to do:
-    # forward 2 GEMMs, dK/dV 4 GEMMs (S, dP, dV, dK), dQ 3 GEMMs (S, dP, dQ); one
+    # Dominant kernel of the step (the kernels the default step launches) and the GEMM work it is
+    # required to do: forward 2 GEMMs, dK/dV 4 GEMMs (S, dP, dV, dK), dQ from stored dS 1 GEMM; one
     # causal GEMM = 2*B*H*S^2*D*0.5 FLOP.
     gemm = 2.0 * B * H * S * S * D * (0.5 if causal else 1.0)
-    kernels = {'fwd_kernel': (r_fwd, 2 * gemm), 'bwd_dkdv_kernel': (r_dkdv, 4 * gemm),
-               'bwd_dq_kernel': (r_dq, 3 * gemm)}
+    kernels = {'fwd_kernel': (r_fwd, 2 * gemm), 'bwd_dkdv_kernel (storing dS)': (r_dkdv_s, 4 * gemm),
+               'bwd_dqs_kernel': (r_dqs, 1 * gemm)}
     dom = max(kernels, key=lambda kname: kernels[kname][0]['mean'])
     dom_r, dom_fl = kernels[dom]
     dom_ms = dom_r['mean']
-    # the backward as a whole in the reference's convention (5 GEMMs of algorithmic work, 7 executed)
-    # (the dQ kernel computes delta itself and hands it to the dK/dV kernel: two launches)
-    bwd_kernels_ms = r_dkdv['mean'] + r_dq['mean']
+    # the backward as a whole in the reference's convention (5 GEMMs of algorithmic work; 5 executed
+    # when dS is kept, 7 when the dQ kernel recomputes)
+    bwd_kernels_ms = r_prep['mean'] + r_dkdv_s['mean'] + r_dqs['mean']
     elem = 2 * B * H * S * D                                   # bytes of one bf16 activation tensor
+    ds_bytes = 2.0 * B * H * S * S * (0.5 if causal else 1.0)  # one 16-bit dS value per visible (query, key) pair
     algorithmic_bytes = {'fwd_kernel': 4 * elem + 4 * B * H * S,            # Q, K, V in, O out, LSE out
-                         'bwd_dkdv_kernel': 6 * elem + 8 * B * H * S,       # Q, K, V, dO in, dK, dV out, LSE, delta in
-                         'bwd_dq_kernel': 6 * elem + 8 * B * H * S}         # Q, K, V, O, dO in, dQ out, LSE in, delta out
+                         # Q, K, V, dO in, dK, dV out, the two row statistics in, dS out
+                         'bwd_dkdv_kernel (storing dS)': 6 * elem + 8 * B * H * S + ds_bytes,
+                         'bwd_dqs_kernel': 2 * elem + ds_bytes}             # K in, dQ out, dS in
     roofline = {'bound': 'mfma', 'kernel': dom, 'achieved': tf(dom_fl, dom_ms), 'peak': PEAK_BF16_TFLOPS,
                 'unit': 'TFLOP/s', 'frac': tf(dom_fl, dom_ms) / PEAK_BF16_TFLOPS,
                 'traffic': hbm_bytes_from_profile(dom), 'algorithmic_bytes': algorithmic_bytes[dom],
                 'avg_ms': dom_ms, 'median_ms': dom_r['median'], 'flop_per_launch': dom_fl,
                 'frac_ref_convention': tf(f_bwd, bwd_kernels_ms) / PEAK_BF16_TFLOPS,
                 'frac_ref_convention_note': 'whole split backward: 2.5 x forward FLOP (5 GEMMs) over the summed '
-                                            'mean durations of its two kernels (dQ, which also computes '
-                                            'delta, then dK/dV); frac counts the GEMMs the dominant kernel '
-                                            'executes'}
+                                            'mean durations of its three kernels (delta and row statistics, '
+                                            'dK/dV writing dS, dQ from dS); frac counts the GEMMs the dominant '
+                                            'kernel executes'}
 
     out = {
         'metric': 'attn fwd/bwd TFLOPS and % bf16 MFMA peak, B4 H32 S4096 D128 causal, 1 GPU',
@@ -319,8 +330,14 @@ def main():
         'timing': 'per launch: 512 MiB zeroed before it, warm-up >= 25 ms, >= 100 ms of launches, HIP events, '
                   'median (p20, p80); value/ms_per_step: K back-to-back steps between synchronisations',
         'fwd': row(f_fwd, r_fwd),
-        'bwd_split': row(f_bwd, r_split, {'kernels_ms': {'bwd_dq_with_delta': r_dq['median'], 'bwd_dkdv': r_dkdv['median'],
-                                                         'bwd_preprocess_standalone_not_launched': r_pre['median']}}),
+        'bwd_split': row(f_bwd, r_split, {'kernels_ms': {'delta_and_row_statistics': r_prep['median'],
+                                                         'bwd_dkdv_storing_ds': r_dkdv_s['median'],
+                                                         'bwd_dq_from_ds': r_dqs['median']},
+                                          'workspace_bytes': ds_bytes * 2 if causal else ds_bytes}),
+        'bwd_split_recompute': row(f_bwd, r_recomp, {'kernels_ms': {'bwd_dq_with_delta': r_dq['median'],
+                                                                    'bwd_dkdv': r_dkdv['median'],
+                                                                    'bwd_preprocess_standalone_not_launched': r_pre['median']},
+                                                     'note': 'workspace limit 0: the dQ kernel recomputes S and dP (7 GEMMs)'}),
         'bwd_fused': row(f_bwd, r_fused),
         'roofline': roofline,
     }
@@ -345,7 +362,6 @@ def main():
         sm4 = 1.0 / math.sqrt(128)
 
         def fwd4():
-            atomic.zero_()
             assert flash.attn_fwd_compact_varlen(q4, k4, v4, None, cuq, cuq, mx, mx, sm4, L4, o4, 0.0, null, null, 0,
                                                  null, null, None, True, atomic) == ok
 
@@ -376,7 +392,6 @@ def main():
         sm5 = 1.0 / math.sqrt(D5)
 
         def fwd5():
-            atomic.zero_()
             assert flash.attn_fwd(q5, k5, v5, b5, sm5, L5, o5, 0.1, seed5, off5, 0, so5, oo5, None, (1024, 0), atomic) == ok
 
         def bwd5(with_db):

@@ -304,7 +304,10 @@ FA_API int fa_trim_workspace(void);
 
 /* One kernel of the backward only: kernel_slot 0 = delta (bwd_preprocess), 1 = dK/dV
  * (reads delta), 2 = dQ (16-bit types up to head dim 256: computes delta and writes it;
- * otherwise reads it), 3 = fused.  Slots 0-2 need an eager delta buffer in params->D.  Stands in
+ * otherwise reads it), 3 = fused; of the backward that keeps dS in the library's workspace (calls
+ * that qualify for it, else FA_ERROR_NOT_SUPPORTED): 4 = delta and the prepared row statistics,
+ * 5 = dK/dV writing dS, 6 = dQ from the stored dS (what slot 5 left in the workspace).  All slots
+ * but 3 need an eager delta buffer in params->D.  Stands in
  * for the per-kernel selection of the reference's tuning interface
  * (attn_options::KernelSlot, include/aotriton/flash.h:46-60; include/aotriton/cpp_tune.h)
  * and is what the benchmark uses to time kernels one at a time. */
