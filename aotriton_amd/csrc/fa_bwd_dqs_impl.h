@@ -110,8 +110,7 @@ __device__ __forceinline__ void dqs_item(const BwdArgs& a, const int h, const in
       rows = rows < BN ? rows : BN;
       rows = j <= j1 ? rows : 0;
       const T* kt = kbase + (int64_t)j * BN * a.sk.s;
-      const auto k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0,
-                                                          rows > 0 ? ((rows - 1) * (int)a.sk.s + d_qk) * 2 : 0, 0x00020000);
+      const auto k_rs = wave_rsrc(kt, rows > 0 ? ((rows - 1) * (int)a.sk.s + d_qk) * 2 : 0);
 #pragma unroll
       for (int k = 0; k < CH; ++k)
         kreg[k] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff, k * k_soff, 0));
@@ -132,7 +131,7 @@ __device__ __forceinline__ void dqs_item(const BwdArgs& a, const int h, const in
       const int nt = j / SPT, kw0 = (j % SPT) * KWS;
       const char* tile = ws_head + ((int64_t)nt * a.ds_ntq + pm) * DT::BYTES;
       // a wave that has nothing to fetch at this step reads through an empty descriptor: zeros, no traffic
-      const auto rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile), 0, active(j) ? DT::BYTES : 0, 0x00020000);
+      const auto rs = wave_rsrc(tile, active(j) ? DT::BYTES : 0);
 #pragma unroll
       for (int i = 0; i < NCK; ++i)
         dsr[R][i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(

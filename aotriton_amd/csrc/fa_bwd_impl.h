@@ -242,7 +242,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   auto ds_slot_of = [](int t) { return TS >= kDsSlots ? t * kDsSlots / TS : 2 * t + 1; };
   auto store_ds_slot = [&](char* tile, int slot) {
     if constexpr (kStoreDs) {
-      const auto rs = __builtin_amdgcn_make_buffer_rsrc(tile, 0, tile != nullptr ? DT::BYTES : 0, 0x00020000);
+      const auto rs = wave_rsrc(tile, tile != nullptr ? DT::BYTES : 0);
 #pragma unroll
       for (int t = 0; t < TS; ++t)
         if (ds_slot_of(t) == slot)
@@ -343,24 +343,20 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
              (int64_t)(hk * group + g) * a.sb_h + (int64_t)br.lo * BM * a.sb_m + (int64_t)n0 * a.sb_n;
       bb_tile = bb;
       b_rows = rows;
-      b_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(bb), 0,
-                                               any && bias_lds ? ((rows - 1) * (int)a.sb_m + b_cols) * 2 : 0, 0x00020000);
+      b_rs = wave_rsrc(bb, any && bias_lds ? ((rows - 1) * (int)a.sb_m + b_cols) * 2 : 0);
       if (live) bb += (int64_t)BM * a.sb_m;
     }
-    q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qb), 0, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0,
-                                             0x00020000);
-    do_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(dob), 0,
-                                              any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0, 0x00020000);
+    q_rs = wave_rsrc(qb, any ? ((rows - 1) * (int)a.sq.s + d_qk) * 2 : 0);
+    do_rs = wave_rsrc(dob, any ? ((rows - 1) * (int)a.sdo.s + d_v) * 2 : 0);
     if (kInlineDelta)
-      o_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(ob), 0,
-                                               any ? ((rows - 1) * (int)a.so.s + d_v) * 2 : 0, 0x00020000);
+      o_rs = wave_rsrc(ob, any ? ((rows - 1) * (int)a.so.s + d_v) * 2 : 0);
     if constexpr (kStoreDs) {
       // the prepared statistics (L log2e; -delta, or delta with dropout) go straight into the stage:
       // no register load in the loop, hence no wait of the compiler's for one at the end of a tile
       // (16 bytes per lane: BM / 4 lanes of wave 0 fetch each array)
       if (tid < BM / 4) {
-        const auto l_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(lse_b), 0, rows * 4, 0x00020000);
-        const auto d_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(delta_b), 0, rows * 4, 0x00020000);
+        const auto l_rs = wave_rsrc(lse_b, rows * 4);
+        const auto d_rs = wave_rsrc(delta_b, rows * 4);
         char* st = stage_ptr(f_stage) + 2 * SM::TILE_BYTES;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(l_rs, (lds_ptr_t)st, 16, lane * 16, 0, 0, 0);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(d_rs, (lds_ptr_t)(st + BM * 4), 16, lane * 16, 0, 0, 0);
@@ -782,8 +778,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const T* vt = reinterpret_cast<const T*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                   (int64_t)(si.k_start + n0) * a.sv.s;
     const int rows = si.seqlen_k - n0 < BN ? si.seqlen_k - n0 : BN;
-    const auto v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0,
-                                                        ((rows - 1) * (int)a.sv.s + d_v) * 2, 0x00020000);
+    const auto v_rs = wave_rsrc(vt, ((rows - 1) * (int)a.sv.s + d_v) * 2);
     constexpr int VCH = BN * D / 8 / NT;
 #pragma unroll
     for (int i = 0; i < VCH; ++i) {
@@ -1095,10 +1090,8 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
     int rows = rows_left < BN ? rows_left : BN;
     rows = live ? rows : 0;
     const bool any = rows > 0;
-    k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, any ? ((rows - 1) * (int)a.sk.s + d_qk) * 2 : 0,
-                                             0x00020000);
-    v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, any ? ((rows - 1) * (int)a.sv.s + d_v) * 2 : 0,
-                                             0x00020000);
+    k_rs = wave_rsrc(kt, any ? ((rows - 1) * (int)a.sk.s + d_qk) * 2 : 0);
+    v_rs = wave_rsrc(vt, any ? ((rows - 1) * (int)a.sv.s + d_v) * 2 : 0);
     if (live) { kt += k_step; vt += v_step; rows_left -= BN; }
   };
   constexpr int FETCH_PIECES = 2 * CH;

@@ -111,8 +111,7 @@ struct TileFetch {
   op_t reg[CH];
   __device__ __forceinline__ void load(const T* tile, int rows, int64_t row_stride, int cols, int tid) {
     const int r0 = tid >> 6, cc0 = tid & 63;
-    const auto rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(tile), 0,
-                                                      rows > 0 ? ((rows - 1) * (int)row_stride + cols) * 2 : 0, 0x00020000);
+    const auto rs = wave_rsrc(tile, rows > 0 ? ((rows - 1) * (int)row_stride + cols) * 2 : 0);
     const int voff = cc0 * 8 < cols ? r0 * (int)row_stride * 2 + cc0 * 16 : kVoffOutOfRange;
 #pragma unroll
     for (int i = 0; i < CH; ++i)

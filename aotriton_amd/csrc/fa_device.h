@@ -149,6 +149,23 @@ __device__ __forceinline__ typename Traits<T>::op_t swz_read_tr(const char* tile
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// The one place where a buffer descriptor is built.  Every argument passes through
+// v_readfirstlane: the descriptor is then uniform for the compiler whatever it was derived from.
+// A descriptor built from a value the compiler takes for divergent (threadIdx.x >> 6, say, which
+// is the same in all lanes of a wave without the compiler knowing it) makes it wrap every access
+// in a loop over the distinct descriptors, and hipcc 7.2 has placed a register spill into the exit
+// block of such a loop, where no lane is enabled: the store is lost and the reload returns what the
+// slot held before.  On values that are uniform already the three instructions fold away.
+// bytes: length of the range, accesses past it read zero / write nothing.
+template <typename P>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_rsrc(P* base, int bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>((uint64_t)hi << 32 | lo), 0,
+                                           __builtin_amdgcn_readfirstlane(bytes), 0x00020000);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

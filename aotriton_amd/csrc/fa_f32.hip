@@ -107,8 +107,7 @@ struct TileFetch {
   f32x4 reg[CH];
   __device__ __forceinline__ void load(const float* tile, int rows, int64_t row_stride, int cols, int tid) {
     const int r0 = tid / LPR, cc0 = tid % LPR;
-    const auto rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(tile), 0,
-                                                      rows > 0 ? ((rows - 1) * (int)row_stride + cols) * 4 : 0, 0x00020000);
+    const auto rs = wave_rsrc(tile, rows > 0 ? ((rows - 1) * (int)row_stride + cols) * 4 : 0);
     const int voff = cc0 * 4 < cols ? r0 * (int)row_stride * 4 + cc0 * 16 : kVoffOutOfRange;
 #pragma unroll
     for (int i = 0; i < CH; ++i)

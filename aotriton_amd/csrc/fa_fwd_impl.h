@@ -158,10 +158,8 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   int rows_left = si.seqlen_k - br.lo * BN;      // > 0
   auto load_next_tile = [&]() {
     const int rows = rows_left < BN ? rows_left : BN;
-    const auto krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(kt), 0, (rows - 1) * k_row_bytes + d_qk * 2,
-                                                       0x00020000);
-    const auto vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(vt), 0, (rows - 1) * v_row_bytes + d_v * 2,
-                                                       0x00020000);
+    const auto krs = wave_rsrc(kt, (rows - 1) * k_row_bytes + d_qk * 2);
+    const auto vrs = wave_rsrc(vt, (rows - 1) * v_row_bytes + d_v * 2);
 #pragma unroll
     for (int i = 0; i < CH; ++i)
       kreg[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvoff, i * ksoff, 0));
@@ -179,8 +177,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   {
     const T* qw = reinterpret_cast<const T*>(a.q) + (int64_t)si.batch_index * a.sq.z + (int64_t)h * a.sq.h +
                   (int64_t)(si.q_start + q0 + wave_u * 32) * a.sq.s;
-    const auto qrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(qw), 0,
-                                                       wrows > 0 ? ((wrows - 1) * (int)a.sq.s + d_qk) * 2 : 0, 0x00020000);
+    const auto qrs = wave_rsrc(qw, wrows > 0 ? ((wrows - 1) * (int)a.sq.s + d_qk) * 2 : 0);
     const int qvoff = cq * 8 < d_qk ? rq * (int)a.sq.s * 2 + cq * 16 : kVoffOutOfRange;
     op_t qin[32 / RPQ];
 #pragma unroll
@@ -538,8 +535,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
   {
     T* ow = reinterpret_cast<T*>(a.out) + (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h +
             (int64_t)(si.q_start + q0 + wave_u * 32) * a.so.s;
-    const auto ors = __builtin_amdgcn_make_buffer_rsrc(ow, 0, wrows > 0 ? ((wrows - 1) * (int)a.so.s + d_v) * 2 : 0,
-                                                       0x00020000);
+    const auto ors = wave_rsrc(ow, wrows > 0 ? ((wrows - 1) * (int)a.so.s + d_v) * 2 : 0);
     const int ovoff = cq * 8 < d_v ? rq * (int)a.so.s * 2 + cq * 16 : kVoffOutOfRange;
 #pragma unroll
     for (int i = 0; i < 32 / RPQ; ++i) {

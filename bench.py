@@ -97,6 +97,9 @@ def main():
     ap.add_argument('--tile-entry', default=None, metavar='D,causal,dtype',
                     help='run the forward, dK/dV and dQ kernels of one tile-table entry a few times and print their '
                          'times (for profiler runs), e.g. 64,1,bf16: B = 4, H = 4096 / D, S = 4096; D up to 512, dtype bf16, fp16 or fp32')
+    ap.add_argument('--only', default=None, choices=['c4', 'c5'],
+                    help='run only the forward and the backward of configuration 4 (packed sequences) or 5 (D=256, window + '
+                         'bias + dropout) a few times and print their times (for profiler runs)')
     ap.add_argument('--mfma-peak', action='store_true',
                     help='only measure what the matrix pipe sustains (register-only MFMA loop, constant '
                          'and random operands) and print that as one JSON line')
@@ -147,6 +150,83 @@ def main():
         t = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
         q = lambda p: t[min(n - 1, int(p * n))]
         return {'median': q(0.5), 'p20': q(0.2), 'p80': q(0.8), 'mean': sum(t) / n, 'reps': n}
+
+    def make_c4():
+        """(forward, backward, forward FLOP, description) of configuration 4"""
+        rng = np.random.default_rng(1234)
+        lens = rng.integers(256, 8193, size=16)
+        cu = np.zeros(17, dtype=np.int32)
+        cu[1:] = np.cumsum(lens)
+        T, Hq, Hk = int(cu[-1]), 32, 8
+        gg = torch.Generator(device=dev).manual_seed(1234)
+        mk = lambda h: torch.randn(1, T, h, 128, device=dev, dtype=torch.float32, generator=gg).to(torch.bfloat16).transpose(1, 2)
+        q4, k4, v4, do4 = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
+        o4, dq4, dk4, dv4 = torch.empty_like(q4), torch.empty_like(q4), torch.empty_like(k4), torch.empty_like(v4)
+        L4 = torch.empty(Hq, T, device=dev, dtype=torch.float32)
+        d4 = torch.empty_like(L4)
+        cuq = torch.from_numpy(cu).to(dev)
+        mx = int(lens.max())
+        sm4 = 1.0 / math.sqrt(128)
+
+        def fwd4():
+            assert flash.attn_fwd_compact_varlen(q4, k4, v4, None, cuq, cuq, mx, mx, sm4, L4, o4, 0.0, null, null, 0,
+                                                 null, null, None, True, atomic) == ok
+
+        def bwd4():
+            assert flash.attn_bwd_compact_varlen(q4, k4, v4, cuq, cuq, mx, mx, None, sm4, o4, do4, dq4, dk4, dv4, None,
+                                                 L4, d4, 0.0, null, null, 0, True) == ok
+
+        fl4 = sum(4.0 * Hq * float(n) ** 2 * 128 * 0.5 for n in lens)
+        return fwd4, bwd4, fl4, (f'GQA Hq=32 Hkv=8 D=128 bf16 causal, 16 packed sequences U[256,8192] (seed 1234), '
+                                 f'{T} tokens, THD storage')
+
+    def make_c5():
+        """(forward, backward(with_db), forward FLOP, description) of configuration 5"""
+        gg = torch.Generator(device=dev).manual_seed(1234)
+        B5, H5, S5, D5 = 2, 16, 8192, 256
+        rn5 = lambda *s, sc=1.0: (torch.randn(*s, device=dev, dtype=torch.float32, generator=gg) * sc).to(torch.float16)
+        q5, k5, v5, do5 = (rn5(B5, H5, S5, D5) for _ in range(4))
+        b5 = torch.empty(B5, H5, S5, S5, device=dev, dtype=torch.float16)
+        for i in range(B5):
+            for h in range(H5):
+                b5[i, h] = rn5(S5, S5, sc=0.5)
+        o5, dq5, dk5, dv5 = torch.empty_like(q5), torch.empty_like(q5), torch.empty_like(k5), torch.empty_like(v5)
+        db5 = torch.empty_like(b5)
+        L5 = torch.empty(B5 * H5, S5, device=dev, dtype=torch.float32)
+        d5 = torch.empty_like(L5)
+        u64 = lambda x: torch.tensor([x], device=dev, dtype=torch.uint64)
+        seed5, off5, so5, oo5 = u64(0x1234), u64(0), u64(0), u64(0)
+        sm5 = 1.0 / math.sqrt(D5)
+
+        def fwd5():
+            assert flash.attn_fwd(q5, k5, v5, b5, sm5, L5, o5, 0.1, seed5, off5, 0, so5, oo5, None, (1024, 0), atomic) == ok
+
+        def bwd5(with_db):
+            assert flash.attn_bwd(q5, k5, v5, b5, sm5, o5, do5, dq5, dk5, dv5, db5 if with_db else None, None, L5, d5,
+                                  0.1, so5, oo5, 0, (1024, 0)) == ok
+
+        fl5 = 4.0 * B5 * H5 * D5 * 7872000.0          # visible (query, key) pairs per head: sum_i (min(i, 1024) + 1)
+        return fwd5, bwd5, fl5, ('B=2 H=16 S=8192 D=256 fp16, window (1024, 0), bias (B,H,S,S) ~ N(0,0.5), dropout 0.1 '
+                                 'seed 0x1234 offset 0')
+
+    if args.only:
+        null = torch.empty([0], device=dev, dtype=torch.uint64)
+        atomic = torch.zeros([1], device=dev, dtype=torch.int32)
+        f, b, fl, work = make_c4() if args.only == 'c4' else make_c5()
+        runs = {'fwd': f, 'bwd': b} if args.only == 'c4' else {'fwd': f, 'bwd_no_db': lambda: b(False)}
+        res = {}
+        for name, fn in runs.items():
+            fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                fn()
+            e1.record()
+            e1.synchronize()
+            res[name + '_ms'] = e0.elapsed_time(e1) / 3
+        print(json.dumps({'only': args.only, 'workload': work, 'forward_flop': fl, **res}))
+        return
 
     if args.tile_entry:
         d_s, c_s, t_s = args.tile_entry.split(',')
@@ -346,68 +426,19 @@ def main():
         del q, k, v, do, o, dq, dk, dv
         torch.cuda.empty_cache()
         # --- configuration 4: GQA, 16 packed sequences U[256, 8192], causal, bf16, D=128 -------------
-        rng = np.random.default_rng(seed)
-        lens = rng.integers(256, 8193, size=16)
-        cu = np.zeros(17, dtype=np.int32)
-        cu[1:] = np.cumsum(lens)
-        T, Hq, Hk = int(cu[-1]), 32, 8
-        gg = torch.Generator(device=dev).manual_seed(seed)
-        mk = lambda h: torch.randn(1, T, h, 128, device=dev, dtype=torch.float32, generator=gg).to(torch.bfloat16).transpose(1, 2)
-        q4, k4, v4, do4 = mk(Hq), mk(Hk), mk(Hk), mk(Hq)
-        o4, dq4, dk4, dv4 = torch.empty_like(q4), torch.empty_like(q4), torch.empty_like(k4), torch.empty_like(v4)
-        L4 = torch.empty(Hq, T, device=dev, dtype=torch.float32)
-        d4 = torch.empty_like(L4)
-        cuq = torch.from_numpy(cu).to(dev)
-        mx = int(lens.max())
-        sm4 = 1.0 / math.sqrt(128)
-
-        def fwd4():
-            assert flash.attn_fwd_compact_varlen(q4, k4, v4, None, cuq, cuq, mx, mx, sm4, L4, o4, 0.0, null, null, 0,
-                                                 null, null, None, True, atomic) == ok
-
-        def bwd4():
-            assert flash.attn_bwd_compact_varlen(q4, k4, v4, cuq, cuq, mx, mx, None, sm4, o4, do4, dq4, dk4, dv4, None,
-                                                 L4, d4, 0.0, null, null, 0, True) == ok
-
-        fl4 = sum(4.0 * Hq * float(s) ** 2 * 128 * 0.5 for s in lens)
-        out['c4'] = {'workload': f'GQA Hq=32 Hkv=8 D=128 bf16 causal, 16 packed sequences U[256,8192] (seed {seed}), '
-                                 f'{T} tokens, THD storage',
-                     'fwd': row(fl4, do_bench(fwd4)), 'bwd_split': row(2.5 * fl4, do_bench(bwd4))}
-        del q4, k4, v4, do4, o4, dq4, dk4, dv4
+        fwd4, bwd4, fl4, work4 = make_c4()
+        out['c4'] = {'workload': work4, 'fwd': row(fl4, do_bench(fwd4)), 'bwd_split': row(2.5 * fl4, do_bench(bwd4))}
+        del fwd4, bwd4
         torch.cuda.empty_cache()
         # --- configuration 5: B2 H16 S8192 D256 fp16, window (1024, 0) + bias + dropout 0.1 ----------
-        B5, H5, S5, D5 = 2, 16, 8192, 256
-        rn5 = lambda *s, sc=1.0: (torch.randn(*s, device=dev, dtype=torch.float32, generator=gg) * sc).to(torch.float16)
-        q5, k5, v5, do5 = (rn5(B5, H5, S5, D5) for _ in range(4))
-        b5 = torch.empty(B5, H5, S5, S5, device=dev, dtype=torch.float16)
-        for i in range(B5):
-            for h in range(H5):
-                b5[i, h] = rn5(S5, S5, sc=0.5)
-        o5, dq5, dk5, dv5 = torch.empty_like(q5), torch.empty_like(q5), torch.empty_like(k5), torch.empty_like(v5)
-        db5 = torch.empty_like(b5)
-        L5 = torch.empty(B5 * H5, S5, device=dev, dtype=torch.float32)
-        d5 = torch.empty_like(L5)
-        u64 = lambda x: torch.tensor([x], device=dev, dtype=torch.uint64)
-        seed5, off5, so5, oo5 = u64(0x1234), u64(0), u64(0), u64(0)
-        sm5 = 1.0 / math.sqrt(D5)
-
-        def fwd5():
-            assert flash.attn_fwd(q5, k5, v5, b5, sm5, L5, o5, 0.1, seed5, off5, 0, so5, oo5, None, (1024, 0), atomic) == ok
-
-        def bwd5(with_db):
-            assert flash.attn_bwd(q5, k5, v5, b5, sm5, o5, do5, dq5, dk5, dv5, db5 if with_db else None, None, L5, d5,
-                                  0.1, so5, oo5, 0, (1024, 0)) == ok
-
-        fl5 = 4.0 * B5 * H5 * D5 * 7872000.0          # visible (query, key) pairs per head: sum_i (min(i, 1024) + 1)
-        out['c5'] = {'workload': 'B=2 H=16 S=8192 D=256 fp16, window (1024, 0), bias (B,H,S,S) ~ N(0,0.5), dropout 0.1 '
-                                 'seed 0x1234 offset 0',
+        fwd5, bwd5, fl5, work5 = make_c5()
+        out['c5'] = {'workload': work5,
                      'fwd': row(fl5, do_bench(fwd5, max_reps=100)),
                      'bwd_split_no_db': row(2.5 * fl5, do_bench(lambda: bwd5(False), max_reps=60)),
                      'bwd_split_with_db': row(2.5 * fl5, do_bench(lambda: bwd5(True), max_reps=60),
                                               {'note': 'dB is a dense (B,H,S,S) tensor: 4 GiB written, zeros outside the band'})}
-        del q5, k5, v5, do5, b5, db5
+        del fwd5, bwd5
         torch.cuda.empty_cache()
-
         # --- the two other kernel families: head dim 512 (bf16) and fp32 tensors, causal ---------------
         def family(Bx, Hx, Sx, Dx, dt, peak):
             rnx = lambda: torch.randn(Bx, Hx, Sx, Dx, device=dev, dtype=torch.float32, generator=gg).to(dt)

@@ -260,3 +260,30 @@ def test_v2_positional_entry_points_validate_before_any_launch():
                                       None, 0, None, None, None, True, None, s) == E.hipErrorInvalidValue
     assert v2.attn_bwd_compact_varlen(mk(q), mk(k), mk(v), mk(cu), mk(cu), 40, 40, None, 0.1, mk(o), mk(o), mk(q),
                                       mk(k), mk(v), None, mk(L), None, 0.0, None, None, 0, True, s) == E.hipErrorInvalidValue
+
+
+def test_buffer_descriptors_are_built_in_one_place():
+    """Every buffer descriptor of the kernels comes from wave_rsrc (fa_device.h), which makes its
+    arguments wave-uniform for the compiler.  A descriptor built anywhere else can be taken for
+    divergent; the compiler then loops over the distinct descriptors around every access, and a
+    register spilled next to such a loop has been stored with no lane enabled (wrong results now
+    and then, no error).  Source check: the builtin appears once, inside the helper."""
+    import glob
+    import re
+    csrc = os.path.join(ROOT, 'aotriton_amd', 'csrc')
+    uses = []
+    for path in sorted(glob.glob(os.path.join(csrc, '*.h')) + glob.glob(os.path.join(csrc, '*.hip')) +
+                       glob.glob(os.path.join(csrc, '*.cpp'))):
+        text = open(path).read()
+        text = re.sub(r'//[^\n]*', '', text)                    # comments may name the builtin
+        for m in re.finditer(r'__builtin_amdgcn_make_buffer_rsrc', text):
+            uses.append((os.path.basename(path), text.count('\n', 0, m.start()) + 1))
+    assert [u[0] for u in uses] == ['fa_device.h'], f'buffer descriptors built outside wave_rsrc: {uses}'
+    dev = open(os.path.join(csrc, 'fa_device.h')).read()
+    body = dev[dev.index('wave_rsrc(P* base, int bytes)'):]
+    body = body[:body.index('\n}\n')]
+    assert body.count('__builtin_amdgcn_readfirstlane') == 3 and '__builtin_amdgcn_make_buffer_rsrc' in body
+    # descriptors of other origin would have to be typed somewhere: the type's name appears only where one is held
+    for path in glob.glob(os.path.join(csrc, '*')):
+        if os.path.isfile(path) and path.endswith(('.h', '.hip', '.cpp')):
+            assert 'amdgcn_make_buffer_rsrc(' not in re.sub(r'//[^\n]*', '', open(path).read()) or path.endswith('fa_device.h')

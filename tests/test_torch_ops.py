@@ -132,10 +132,12 @@ def test_sdpa_dropout_follows_torch_generator():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize('dropout_p', [0.0, 0.2])
-def test_forward_and_backward_replay_from_a_hip_graph(dropout_p):
-    """The operators allocate nothing themselves and launch on the caller's stream, so a
-    forward + backward can be captured into a graph.  Every replay (with eager work and
-    synchronisation between replays) must reproduce the eager result bit for bit."""
+def test_forward_and_backward_replay_from_a_hip_graph(dropout_p, recomputing_backward):
+    """The operators launch on the caller's stream and, under stream capture, allocate nothing (the
+    backward then leaves its dS workspace alone and recomputes), so a forward + backward can be
+    captured into a graph.  Every replay (with eager work and synchronisation between replays)
+    must reproduce the eager result bit for bit; the eager runs use the recomputing kernels too,
+    which is what a capture records."""
     from aotriton_amd import torch_ops  # noqa: F401
     q, k, v, _, do = _inputs(B=2, Hq=4, Hk=2, Sq=300, Sk=300, D=128, seed=9)
     sm = 1.0 / math.sqrt(128)

@@ -1,6 +1,8 @@
 """fa_attn_bwd_noalloc (delta in the library's own device array, nothing allocated) against
 fa_attn_bwd with the split backend, through the C ABI: bit-identical dQ, dK, dV on two calls in
-a row, the second with a smaller input, and the size limit."""
+a row, the second with a smaller input, and the size limit.  fa_attn_bwd runs with its dS
+workspace switched off here: the entry point that allocates nothing uses the recomputing kernels,
+and only the same kernels give the same bits."""
 import math
 
 import pytest
@@ -35,16 +37,23 @@ def _run_pair(B, Hq, Hk, Sq, Sk, D, dtype, causal, seed):
     params = attn_bwd_params()
     flash._fill_bwd(params, q, k, v, None, sm, o, do, got[0], got[1], got[2], None, None, L, None, 0.0, null, null, 0,
                     causal)
-    before = torch.cuda.memory_allocated()
+    assert attn_bwd_noalloc(params, attn_bwd_params.kVersion, flash._stream()) == ok      # warm-up: symbol lookup, LDS limits
+    torch.cuda.synchronize()
+    for t in got:
+        t.fill_(float('nan'))
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     assert attn_bwd_noalloc(params, attn_bwd_params.kVersion, flash._stream()) == ok
     torch.cuda.synchronize()
+    # neither torch's allocator nor the device itself (hipMemGetInfo: a hipMalloc inside the library would show) gave memory
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before
     for name, g, r in zip(('dq', 'dk', 'dv'), got, ref):
         assert not torch.isnan(g.float()).any(), name
         assert torch.equal(g, r), name
 
 
-def test_two_calls_in_a_row_second_smaller():
+def test_two_calls_in_a_row_second_smaller(recomputing_backward):
     _run_pair(2, 4, 2, 1000, 777, 128, torch.bfloat16, True, seed=11)
     _run_pair(1, 2, 2, 130, 200, 64, torch.float16, False, seed=12)
 
