@@ -180,7 +180,65 @@ void ws_release(int dev, hipStream_t stream) {
   g_ws_mutex.unlock();
 }
 
+// A call that holds the workspace (the repacking layer below) hands a part of it to the call it
+// makes: that call must neither lock nor grow the buffer.
+struct NestedWorkspace { bool active = false; void* ptr = nullptr; size_t bytes = 0; };
+thread_local NestedWorkspace t_ws_nested;
+
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+}
+
 bool is_16bit(int dt) { return dt == FA_DTYPE_FLOAT16 || dt == FA_DTYPE_BFLOAT16; }
+
+// ---- packed copies of tensors whose rows are not made of aligned 16-byte pieces ----------------
+// (a head dim or a stride that is no multiple of 8 elements, a base that is not 16-byte aligned).
+// The reference runs any head dim on its tuned kernels by padding it inside them
+// (modules/flash/csrc/attn_fwd.cc:76-82,109, kernel/composed_tensors.py:60-93).  Here such a call
+// gets contiguous copies with the head dim rounded up to a multiple of 8 (zeros in the excess
+// columns, which add nothing to any dot product) in the library's workspace, runs on the MFMA
+// kernels and has its results copied back; without workspace (limit, stream capture) it runs on
+// the element-wise vector-ALU kernels.
+int elem_bytes_of(int dt) { return dt == FA_DTYPE_FLOAT32 ? 4 : 2; }
+
+size_t packed_bytes(const fa_tensor4& t) {
+  const uint64_t dp = (t.sizes[3] + 7) / 8 * 8;
+  const uint64_t n = t.sizes[0] * t.sizes[1] * t.sizes[2] * dp * (uint64_t)elem_bytes_of(t.dtype);
+  return (size_t)((n + 255) & ~(uint64_t)255);
+}
+
+fa_tensor4 packed_view(const fa_tensor4& t, void* ptr) {
+  fa_tensor4 v = t;
+  const uint64_t dp = (t.sizes[3] + 7) / 8 * 8;
+  v.ptr = (t.sizes[0] * t.sizes[1] * t.sizes[2]) != 0 ? ptr : nullptr;
+  v.sizes[3] = dp;
+  v.strides[3] = 1;
+  v.strides[2] = dp;
+  v.strides[1] = t.sizes[2] * dp;
+  v.strides[0] = t.sizes[1] * t.sizes[2] * dp;
+  return v;
+}
+
+hipError_t repack(const fa_tensor4& strided, const fa_tensor4& packed, bool unpack, hipStream_t stream) {
+  if (packed.ptr == nullptr || strided.ptr == nullptr) return hipSuccess;
+  fa::RepackArgs a{};
+  a.strided = strided.ptr; a.packed = packed.ptr;
+  a.s0 = (int64_t)strided.strides[0]; a.s1 = (int64_t)strided.strides[1]; a.s2 = (int64_t)strided.strides[2];
+  a.n0 = (int32_t)strided.sizes[0]; a.n1 = (int32_t)strided.sizes[1]; a.n2 = (int32_t)strided.sizes[2];
+  a.d = (int32_t)strided.sizes[3]; a.dp = (int32_t)packed.sizes[3];
+  return fa::run_repack(elem_bytes_of(strided.dtype), unpack, a, stream);
+}
+
+// bytes of packed copies a call on the element-wise kernels would need instead
+size_t fwd_copies_bytes(const fa_fwd_params* p) {
+  return packed_bytes(p->Q) + packed_bytes(p->K) + packed_bytes(p->V) + packed_bytes(p->Out);
+}
+size_t bwd_copies_bytes(const fa_bwd_params* p) {
+  size_t n = 0;
+  for (const fa_tensor4* t : {&p->Q, &p->K, &p->V, &p->Out, &p->DO, &p->DQ, &p->DK, &p->DV}) n += packed_bytes(*t);
+  return n;
+}
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -503,6 +561,10 @@ int fa_tile_intervals(int32_t causal_type, int32_t window_left, int32_t window_r
 int fa_check_gpu(void* hip_stream) {
   const DeviceInfo* d = device_of_stream(static_cast<hipStream_t>(hip_stream));
   if (d == nullptr || !d->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+  // the address of fa_attn_bwd_noalloc's array is looked up here as well: a first call of that
+  // entry point under stream capture then finds it and makes no call that a capture forbids
+  float* unused = nullptr;
+  (void)scratch_of_device(device_index(d), &unused);
   return FA_SUCCESS;
 }
 
@@ -554,6 +616,12 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   out->backend_index = 0;
   out->head_dim = s.d;
   out->flags = (s.windowed ? 1 : 0) | (s.bias ? 2 : 0) | (s.dropout ? 4 : 0) | (s.num_seqlens != 0 ? 8 : 0);
+  // 32: fa_attn_fwd would run this call on packed copies in the workspace of the current device (the
+  // tile and grid above are those of the element-wise kernels it runs on otherwise)
+  int dev = 0;
+  if (s.elementwise && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices &&
+      (int64_t)fwd_copies_bytes(params) <= ws_limit_bytes(dev))
+    out->flags |= 32;
   return FA_SUCCESS;
 }
 
@@ -615,6 +683,11 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
     if (need > 0 && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices && need <= ws_limit_bytes(dev))
       out->flags |= 16;
   }
+  // 32: fa_attn_bwd would run this call on packed copies in the workspace
+  int dev = 0;
+  if (s.elementwise && hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices &&
+      (int64_t)bwd_copies_bytes(params) <= ws_limit_bytes(dev))
+    out->flags |= 32;
   return FA_SUCCESS;
 }
 
@@ -647,6 +720,34 @@ int fa_attn_fwd(const fa_fwd_params* p, int32_t params_version, void* hip_stream
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   const DeviceInfo* dev = device_of_stream(stream);
   if (dev == nullptr || !dev->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
+
+  if (s.elementwise && !t_ws_nested.active && !stream_is_capturing(stream)) {
+    // packed copies of Q, K, V and Out in the workspace, the MFMA kernels on those, Out copied back
+    const fa_tensor4* in[3] = {&p->Q, &p->K, &p->V};
+    const size_t need = fwd_copies_bytes(p);
+    void* base = nullptr;
+    if ((int64_t)need <= ws_limit_bytes(device_index(dev)) && ws_acquire(device_index(dev), need, stream, &base) == hipSuccess) {
+      fa_fwd_params p2 = *p;
+      char* at = static_cast<char*>(base);
+      fa_tensor4* to[3] = {&p2.Q, &p2.K, &p2.V};
+      hipError_t err = hipSuccess;
+      for (int i = 0; i < 3 && err == hipSuccess; ++i) {
+        *to[i] = packed_view(*in[i], at);
+        at += packed_bytes(*in[i]);
+        err = repack(*in[i], *to[i], false, stream);
+      }
+      p2.Out = packed_view(p->Out, at);
+      int rc = (int)err;
+      if (err == hipSuccess) {
+        t_ws_nested = NestedWorkspace{true, nullptr, 0};
+        rc = fa_attn_fwd(&p2, params_version, hip_stream, options);
+        t_ws_nested = NestedWorkspace{};
+      }
+      if (rc == FA_SUCCESS) rc = (int)repack(p->Out, p2.Out, true, stream);
+      ws_release(device_index(dev), stream);
+      return rc;
+    }
+  }
 
   fa::FwdArgs a{};
   a.q = p->Q.ptr; a.k = p->K.ptr; a.v = p->V.ptr; a.bias = p->B.ptr;
@@ -735,6 +836,45 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
   const DeviceInfo* dev = device_of_stream(stream);
   if (dev == nullptr || !dev->is_gfx950) return FA_ERROR_NO_BINARY_FOR_GPU;
 
+  if (s.elementwise && kernel_slot < 0 && !own_delta && !t_ws_nested.active && !stream_is_capturing(stream)) {
+    // packed copies of the eight activation tensors, the MFMA kernels on those, dQ, dK, dV copied back;
+    // the packed call gets the rest of the buffer for its own use (dS)
+    const fa_tensor4* all[8] = {&p->Q, &p->K, &p->V, &p->Out, &p->DO, &p->DQ, &p->DK, &p->DV};
+    const size_t copies = bwd_copies_bytes(p);
+    fa_bwd_params p2 = *p;
+    fa_tensor4* to[8] = {&p2.Q, &p2.K, &p2.V, &p2.Out, &p2.DO, &p2.DQ, &p2.DK, &p2.DV};
+    for (int i = 0; i < 8; ++i) *to[i] = packed_view(*all[i], reinterpret_cast<void*>(uintptr_t(256)));   // shapes first
+    Shape s2{};
+    int be2 = 0;
+    int64_t inner = 0;
+    if (validate_bwd(&p2, params_version, options, &s2, &be2) == FA_SUCCESS && be2 == 0) {
+      int ntq = 0, ntk = 0;
+      int64_t ds_bytes = 0, stat_bytes = 0;
+      inner = ds_workspace_need(&p2, s2, &ntq, &ntk, &ds_bytes, &stat_bytes);
+      if ((int64_t)copies + inner > ws_limit_bytes(device_index(dev))) inner = 0;
+    }
+    const size_t need = copies + (size_t)inner;
+    void* base = nullptr;
+    if ((int64_t)need <= ws_limit_bytes(device_index(dev)) && ws_acquire(device_index(dev), need, stream, &base) == hipSuccess) {
+      char* at = static_cast<char*>(base);
+      hipError_t err = hipSuccess;
+      for (int i = 0; i < 8; ++i) {
+        *to[i] = packed_view(*all[i], at);
+        at += packed_bytes(*all[i]);
+        if (i < 5 && err == hipSuccess) err = repack(*all[i], *to[i], false, stream);
+      }
+      int rc = (int)err;
+      if (err == hipSuccess) {
+        t_ws_nested = NestedWorkspace{true, inner > 0 ? at : nullptr, (size_t)inner};
+        rc = attn_bwd_impl(&p2, params_version, hip_stream, options, kernel_slot, false);
+        t_ws_nested = NestedWorkspace{};
+      }
+      for (int i = 5; i < 8 && rc == FA_SUCCESS; ++i) rc = (int)repack(*all[i], *to[i], true, stream);
+      ws_release(device_index(dev), stream);
+      return rc;
+    }
+  }
+
   fa::BwdArgs a{};
   a.q = p->Q.ptr; a.k = p->K.ptr; a.v = p->V.ptr; a.bias = p->B.ptr;
   a.out = p->Out.ptr; a.dout = p->DO.ptr;
@@ -802,10 +942,18 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);
       return FA_ERROR_NOT_SUPPORTED;
     }
-    if (need > 0 && need <= ws_limit_bytes(device_index(dev))) {
-      hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-      const bool capturing = hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
-      if (!capturing) {
+    const bool nested = t_ws_nested.active;
+    if (nested) {
+      // (the caller holds the buffer and has set a part of it aside)
+      if (need > 0 && (size_t)need <= t_ws_nested.bytes) {
+        ds_ws = t_ws_nested.ptr;
+        a.ds_ntq = ntq;
+        a.ds_ntk = ntk;
+        a.lse_scaled = reinterpret_cast<const float*>(static_cast<char*>(ds_ws) + ds_bytes);
+        a.delta_prep = reinterpret_cast<const float*>(static_cast<char*>(ds_ws) + ds_bytes + stat_bytes);
+      }
+    } else if (need > 0 && need <= ws_limit_bytes(device_index(dev))) {
+      if (!stream_is_capturing(stream)) {
         if (ws_acquire(device_index(dev), (size_t)need, stream, &ds_ws) == hipSuccess) {
           a.ds_ntq = ntq;
           a.ds_ntk = ntk;
@@ -827,7 +975,7 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       if (err == hipSuccess && (ds_slot < 0 || ds_slot == 1))
         err = fa::run_bwd_dkdv(dt, s.d, a, s.windowed, s.bias, s.dropout, stream);
       if (err == hipSuccess && (ds_slot < 0 || ds_slot == 2)) err = fa::run_bwd_dqs(dt, s.d, a, stream);
-      ws_release(device_index(dev), stream);
+      if (!nested) ws_release(device_index(dev), stream);
       if (acquired && lazy->dispose != nullptr) lazy->dispose(lazy);
       return (int)err;
     }

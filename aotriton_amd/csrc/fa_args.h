@@ -88,6 +88,16 @@ struct BwdArgs {
   const float* delta_prep;   // -delta (delta with dropout)
 };
 
+// Copy between a rank-4 tensor of any strides and head dim (unit last stride) and its packed
+// image: contiguous (n0, n1, n2, dp) with dp the head dim rounded up to a multiple of 8, zeros in
+// the excess columns.
+struct RepackArgs {
+  void* strided; void* packed;
+  int64_t s0, s1, s2;     // element strides of the strided tensor
+  int32_t n0, n1, n2;
+  int32_t d, dp;          // columns of the strided tensor / of the packed one
+};
+
 struct EncodedSoftmaxArgs {
   void* r; int64_t s_z, s_h, s_m;
   int32_t batch, heads, seqlen_q, seqlen_k;

@@ -21,6 +21,8 @@ hipError_t run_fwd_d256_padded(int dtype, const FwdArgs& a, bool windowed, bool 
 TileShape fwd_tile_shape(int dtype, int head_dim, bool windowed);
 
 hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s);
+// strided -> packed (unpack false) or packed -> strided (unpack true); elem_bytes 2 or 4
+hipError_t run_repack(int elem_bytes, bool unpack, const RepackArgs& a, hipStream_t s);
 // register-only MFMA loop: the rate the matrix pipe sustains (benchmark aid)
 hipError_t run_mfma_rate(bool random_operands, int grid, int iters, float* out, unsigned long long* clk, hipStream_t s);
 

@@ -42,6 +42,57 @@ hipError_t run_encoded_softmax(const EncodedSoftmaxArgs& a, hipStream_t s) {
   return hipGetLastError();
 }
 
+// Tensors whose rows are not made of aligned 16-byte pieces (a head dim or a stride that is no
+// multiple of 8 elements, an unaligned base) reach the MFMA kernels through a packed copy: one
+// thread moves one group of 8 columns of one row, element by element on the strided side and as one
+// vector on the packed side.  The reference pads such head dims inside its kernels
+// (modules/flash/csrc/attn_fwd.cc:76-82,109); here the padding is a copy in HBM, which costs one
+// pass over the tensor and keeps the kernels' 16-byte staging.
+template <typename E, bool kUnpack>
+__global__ void repack_kernel(const RepackArgs a) {
+  using V = vec<E, 8>;
+  const int groups = a.dp / 8;
+  const int64_t total = (int64_t)a.n0 * a.n1 * a.n2 * groups;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; gid < total; gid += step) {
+    const int g = (int)(gid % groups);
+    const int64_t row = gid / groups;
+    int64_t t = row;
+    const int i2 = (int)(t % a.n2); t /= a.n2;
+    const int i1 = (int)(t % a.n1);
+    const int i0 = (int)(t / a.n1);
+    E* sp = reinterpret_cast<E*>(a.strided) + i0 * a.s0 + i1 * a.s1 + i2 * a.s2 + 8 * g;
+    V* pp = reinterpret_cast<V*>(reinterpret_cast<E*>(a.packed) + row * a.dp + 8 * g);
+    if (kUnpack) {
+      const V v = *pp;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (8 * g + e < a.d) sp[e] = v[e];
+    } else {
+      V v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = 8 * g + e < a.d ? sp[e] : (E)0;
+      *pp = v;
+    }
+  }
+}
+
+hipError_t run_repack(int elem_bytes, bool unpack, const RepackArgs& a, hipStream_t s) {
+  const int64_t total = (int64_t)a.n0 * a.n1 * a.n2 * (a.dp / 8);
+  if (total == 0) return hipSuccess;
+  const int nt = 256;
+  const int64_t nb_all = (total + nt - 1) / nt;
+  dim3 grid((unsigned)(nb_all < (1 << 20) ? nb_all : (1 << 20)));
+  if (elem_bytes == 2) {
+    if (unpack) hipLaunchKernelGGL((repack_kernel<uint16_t, true>), grid, dim3(nt), 0, s, a);
+    else hipLaunchKernelGGL((repack_kernel<uint16_t, false>), grid, dim3(nt), 0, s, a);
+  } else {
+    if (unpack) hipLaunchKernelGGL((repack_kernel<uint32_t, true>), grid, dim3(nt), 0, s, a);
+    else hipLaunchKernelGGL((repack_kernel<uint32_t, false>), grid, dim3(nt), 0, s, a);
+  }
+  return hipGetLastError();
+}
+
 // Register-only loop of v_mfma_f32_32x32x16_bf16 (4 independent accumulators per wave, 8 waves
 // per CU): what the matrix pipe sustains on this machine, on constant operands or on operands
 // with random mantissas (the clock under load depends on the data).  clk[0] = shader cycles,

@@ -166,7 +166,7 @@ def scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.
 # two hooks below give the same effect without touching callers: `sdpa_router()` is a
 # TorchFunctionMode (scoped, composes with torch.compile's tracing of the custom ops), `install()`
 # replaces the attribute on torch.nn.functional for code that cannot be wrapped in a `with`.
-def _routable(query, key, value, attn_mask, dropout_p):
+def _routable(query, key, value, attn_mask, dropout_p, enable_gqa=False):
     ts = (query, key, value)
     if not all(isinstance(t, Tensor) and t.is_cuda and t.dim() == 4 for t in ts):
         return False
@@ -181,7 +181,15 @@ def _routable(query, key, value, attn_mask, dropout_p):
         return False
     if query.shape[1] % max(key.shape[1], 1) or key.shape[1] != value.shape[1]:
         return False
-    if attn_mask is not None and not isinstance(attn_mask, Tensor):
+    # unequal head counts are grouped-query attention only when the caller says so (torch raises otherwise)
+    if query.shape[1] != key.shape[1] and not enable_gqa:
+        return False
+    # what the operators would reject goes to torch, which raises its own error or broadcasts
+    if not (query.shape[0] == key.shape[0] == value.shape[0]) or key.shape[2] != value.shape[2]:
+        return False
+    if not (query.device == key.device == value.device):
+        return False
+    if attn_mask is not None and (not isinstance(attn_mask, Tensor) or attn_mask.device != query.device):
         return False
     if getattr(query, 'is_nested', False) or getattr(key, 'is_nested', False):
         return False
@@ -192,9 +200,8 @@ _torch_sdpa = torch.nn.functional.scaled_dot_product_attention
 
 
 def _dispatch(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None, enable_gqa=False):
-    if _routable(query, key, value, attn_mask, dropout_p):
-        gqa = enable_gqa or query.shape[1] != key.shape[1]
-        return scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal, scale, gqa)
+    if _routable(query, key, value, attn_mask, dropout_p, enable_gqa):
+        return scaled_dot_product_attention(query, key, value, attn_mask, dropout_p, is_causal, scale, enable_gqa)
     return _torch_sdpa(query, key, value, attn_mask=attn_mask, dropout_p=dropout_p, is_causal=is_causal,
                        scale=scale, enable_gqa=enable_gqa)
 

@@ -202,9 +202,17 @@ typedef struct fa_kernel_config {
   int32_t grid[3];
   int32_t backend_index;
   int32_t head_dim;
-  int32_t flags; /* bit0 causal/windowed, bit1 bias, bit2 dropout, bit3 varlen, bit4 (backward) dS kept in HBM */
+  int32_t flags; /* bit0 causal/windowed, bit1 bias, bit2 dropout, bit3 varlen, bit4 (backward) dS kept in HBM, bit5 runs on packed copies */
 } fa_kernel_config;
 
+/* The MFMA kernels read rows made of aligned 16-byte pieces; the test is the same for every element
+ * type: head dims and strides that are multiples of 8 ELEMENTS and 16-byte aligned bases (for fp32
+ * that is stricter than 16 bytes: an fp32 head dim of 12 or 36 fails it).  A call with a tensor that
+ * fails it runs on packed copies (contiguous, head dim rounded up to a multiple of 8 with zeros) that
+ * the library makes in its workspace (fa_set_bwd_workspace_limit below), results copied back: the
+ * MFMA kernels plus one pass over each tensor.  Without workspace (limit too small or 0, a stream
+ * under capture, fa_attn_bwd_kernel, fa_attn_bwd_noalloc) it runs on element-wise vector-ALU
+ * kernels: same results, a few TFLOP/s.  fa_query_*_config sets bit 5 of `flags` for the former. */
 /* v2::flash::check_gpu -- modules/flash/csrc/attn_check.cc:36-46.
  * FA_SUCCESS on gfx950, FA_ERROR_NO_BINARY_FOR_GPU otherwise. */
 FA_API int fa_check_gpu(void* hip_stream);
@@ -213,8 +221,8 @@ FA_API int fa_check_gpu(void* hip_stream);
  * modules/flash/csrc/attn_fwd.cc:48-149.
  * Head dims 1..512 (Dqk of Q and K, Dv of V and Out may differ), rounded up to a built one with the
  * excess columns masked (attn_fwd.cc:76-82).  Tensors whose rows are made of aligned 16-byte pieces
- * (head dims and strides multiples of 8 elements, 16-byte aligned bases) run on the MFMA kernels,
- * anything else on element-wise vector-ALU kernels (same results, a few TFLOP/s).  A bias is
+ * (head dims and strides multiples of 8 elements, 16-byte aligned bases) run on the MFMA kernels as
+ * they are, anything else through packed copies or on element-wise kernels (see above).  A bias is
  * (batch of Q, Hq, Max_seqlen_q, Max_seqlen_k); with cu_seqlens its batch index is the sequence for
  * the padded layout and 0 for packed tokens, rows and columns count from the sequence's start
  * (modules/flash/kernel/fwd_kernel.py:393-395). */
@@ -281,7 +289,10 @@ FA_API int fa_v2_attn_bwd_compact_varlen(
  * process ends); params->D is ignored and nothing is allocated or freed.  It has no
  * counterpart in the reference.  Needs batch * Hq * max_seqlen_q (packed sequences: Hq * tokens)
  * <= FA_NOALLOC_MAX_ROWS, else FA_ERROR_OUT_OF_MEMORY before any launch.  All calls on one GPU
- * share the array: calls that overlap on one GPU (two streams, two threads) race. */
+ * share the array: calls that overlap on one GPU (two streams, two threads) race.  The first call
+ * on a device looks up the device's properties and the array's address (hipGetDeviceProperties,
+ * hipGetSymbolAddress), which a stream capture does not allow: before capturing, call
+ * fa_check_gpu on a stream of that device (it does both lookups) or this entry point once. */
 #define FA_NOALLOC_MAX_ROWS (4 * 1024 * 1024)
 FA_API int fa_attn_bwd_noalloc(const fa_bwd_params* params, int32_t params_version,
                                void* hip_stream);

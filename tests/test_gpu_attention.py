@@ -339,11 +339,12 @@ def test_sampled_strides_bias_layouts_and_masks(i):
 
 
 @pytest.mark.parametrize('D', [7, 23, 37, 53, 67, 73, 89, 113, 149, 179, 211, 241, 203, 300, 509])
-def test_head_dims_that_are_no_multiple_of_8(D):
+def test_head_dims_that_are_no_multiple_of_8(D, with_and_without_workspace):
     """The reference rounds ANY head dim up to a compiled one and masks the excess columns
     (modules/flash/csrc/attn_fwd.cc:76-82,109); its test grid includes the primes below
     (modules/flash/tests/test_forward.py:22,92).  Rows of such tensors are not made of aligned 16-byte
-    pieces and run on the kernels that move single elements (split backend)."""
+    pieces: they reach the MFMA kernels as packed copies in the library's workspace, or, without
+    workspace, run on the kernels that move single elements (split backend)."""
     dtype = [torch.bfloat16, torch.float16, torch.float32][D % 3]
     causal = [False, True, (9, 4)][(D // 3) % 3]
     _run_case(2, 4, 2, 70, 83, D, dtype, causal, dropout_p=0.2 if D % 2 else 0.0, bias=D % 5 == 0, bwd_backend=0, seed=D)
@@ -351,9 +352,9 @@ def test_head_dims_that_are_no_multiple_of_8(D):
 
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize('how', ['base', 'row_stride', 'head_stride'])
-def test_rows_that_are_not_16_byte_aligned(dtype, how):
+def test_rows_that_are_not_16_byte_aligned(dtype, how, with_and_without_workspace):
     """Head dim 64, but a base address that is only element-aligned, a row stride of 65 or a head stride
-    that is no multiple of 8: the same element-wise kernels, same results as the oracle."""
+    that is no multiple of 8: packed copies or the element-wise kernels, same results as the oracle."""
     from aotriton_amd import flash
     from aotriton_amd.autograd import attention, AttentionExtraArgs
     from oracle import fa_ref

@@ -206,3 +206,49 @@ def test_headline_size_with_kept_ds():
     assert (dv_sum - do_sum).abs().max().item() <= 2e-2 * do_sum.abs().max().item()
     # query 0 sees key 0 only: P = 1, dS = dP - delta = 0
     assert a[2][:, :, 0].float().abs().max().item() <= 1e-2
+
+
+def test_packed_copies_take_odd_head_dims_to_the_mfma_kernels():
+    """Head dim 113 (one of the reference's, modules/flash/tests/test_forward.py:22): with workspace the
+    queries report packed copies (bit 5), with the limit at 0 they do not; both give the oracle's results
+    (test_gpu_attention.py) and agree with each other here; the packed way is several times faster."""
+    from aotriton_amd import flash
+    from aotriton_amd.pyaotriton.v3.flash import attn_bwd_params, attn_fwd_params, query_bwd_config, query_fwd_config
+    B, H, S, D = 2, 8, 1024, 113
+    q, k, v, _, do = make_inputs(B, H, H, S, S, D, torch.bfloat16, DEV, seed=5)
+    sm = 1.0 / math.sqrt(D)
+    seed = torch.zeros([1], device=DEV, dtype=torch.uint64)
+    o = torch.empty_like(q)
+    L = torch.empty(B * H, S, device=DEV, dtype=torch.float32)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+
+    def flags():
+        pf, pb = attn_fwd_params(), attn_bwd_params()
+        flash._fill_fwd(pf, q, k, v, None, sm, L, o, 0.0, seed, seed, 0, seed, seed, None, True, atomic)
+        flash._fill_bwd(pb, q, k, v, None, sm, o, do, torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+                        None, None, L, torch.empty_like(L), 0.0, seed, seed, 0, True)
+        ef, cf = query_fwd_config(pf)
+        eb, cb = query_bwd_config(pb, 1)
+        assert ef == eb == flash.hipError_t.hipSuccess
+        return bool(cf.flags & 32), bool(cb.flags & 32), bool(cb.flags & 16)
+
+    def timed(limit):
+        res = _backward(q, k, v, None, do, sm, True, 0.0, limit)      # warms up, grows the buffer
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(3):
+            _backward(q, k, v, None, do, sm, True, 0.0, limit)
+        t1.record()
+        torch.cuda.synchronize()
+        return res, t0.elapsed_time(t1)
+
+    _lib().fa_set_bwd_workspace_limit(-1)
+    assert flags() == (True, True, False)      # dS is kept by the call on the copies, not by this one
+    _lib().fa_set_bwd_workspace_limit(0)
+    assert flags() == (False, False, False)
+    packed, t_packed = timed(-1)
+    plain, t_plain = timed(0)
+    for name, a, b_ in zip(('out', 'L', 'dq', 'dk', 'dv'), packed, plain):
+        assert torch.isfinite(a).all(), name
+        assert (a.float() - b_.float()).abs().max().item() <= 2e-2 * max(1.0, b_.float().abs().max().item()), name
+    assert t_packed * 3 < t_plain, (t_packed, t_plain)

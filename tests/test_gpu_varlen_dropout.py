@@ -135,8 +135,9 @@ def test_many_packed_sequences(nseq, hk, causal):
 
 
 @pytest.mark.parametrize('D,dtype', [(37, torch.bfloat16), (203, torch.float16), (7, torch.float32)])
-def test_compact_varlen_head_dim_no_multiple_of_8(D, dtype):
-    # packed sequences on the element-wise kernels (any head dim, modules/flash/csrc/attn_fwd.cc:76-82)
+def test_compact_varlen_head_dim_no_multiple_of_8(D, dtype, with_and_without_workspace):
+    # packed sequences at any head dim (modules/flash/csrc/attn_fwd.cc:76-82): through packed copies on the
+    # MFMA kernels, and on the element-wise kernels
     _run_varlen_case([5, 0, 70, 33], [9, 64, 41, 33], 4, 2, D, dtype, True, 0, p=0.1)
 
 

@@ -241,3 +241,26 @@ def test_f_sdpa_routes_to_the_library(hook):
         ref = run(lambda a, b, c, **kw: F.scaled_dot_product_attention(a.float(), b.float(), c.float(), **kw))
     for a, b in zip(routed, ref):
         assert (a.float() - b).abs().max().item() < 6e-2
+
+
+def test_router_only_takes_what_the_operators_accept():
+    """unequal head counts without enable_gqa, unequal batch sizes, key and value of different
+    lengths and a mask on another device fall through to torch (which raises its own error or
+    broadcasts); checked on the predicate, with meta tensors standing in for CUDA ones"""
+    from aotriton_amd import torch_ops
+
+    class Fake(torch.Tensor):
+        """a tensor that says it is on the GPU: only the predicate looks at it"""
+        @property
+        def is_cuda(self):
+            return True
+
+    mk = lambda *s: torch.empty(*s, dtype=torch.bfloat16, device='meta').as_subclass(Fake)
+    q, k, v = mk(2, 8, 16, 64), mk(2, 8, 24, 64), mk(2, 8, 24, 64)
+    assert torch_ops._routable(q, k, v, None, 0.0)
+    k2, v2 = mk(2, 2, 24, 64), mk(2, 2, 24, 64)
+    assert not torch_ops._routable(q, k2, v2, None, 0.0)                    # grouped heads, not asked for
+    assert torch_ops._routable(q, k2, v2, None, 0.0, enable_gqa=True)
+    assert not torch_ops._routable(q, mk(1, 8, 24, 64), mk(1, 8, 24, 64), None, 0.0)     # batch sizes
+    assert not torch_ops._routable(q, k, mk(2, 8, 20, 64), None, 0.0)       # key and value lengths
+    assert not torch_ops._routable(q, k, v, torch.zeros(16, 24), 0.0)        # mask elsewhere
