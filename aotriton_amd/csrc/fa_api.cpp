@@ -104,18 +104,18 @@ hipError_t scratch_of_device(int dev, float** out) {
 // Workspace of the backward that keeps dS in HBM between its two kernels: one buffer per device
 // that belongs to the library and only grows (hipMalloc once, then reused: a stream-ordered pool
 // allocation made the host wait for the GPU on every call).  Calls on one device share it: the
-// mutex covers the enqueue, and a call on another stream than the last one first waits (on the
-// GPU) for the event recorded behind the last use.  fa_trim_workspace frees the buffers.
+// device's mutex covers the enqueue, and every call first waits (on the GPU) for the event recorded
+// behind the last use (no work when that was on the same stream; stream handles are not compared:
+// a destroyed stream's handle can come back).  fa_trim_workspace frees the buffers.
 std::atomic<int64_t> g_ws_limit{-1};        // bytes; -1: not set (environment, then default)
 struct Workspace {
   void* ptr = nullptr;
   size_t bytes = 0;
   hipEvent_t done = nullptr;
-  hipStream_t last = nullptr;
   bool used = false;
+  std::mutex mutex;
 };
 Workspace g_ws[kMaxDevices];
-std::mutex g_ws_mutex;
 
 int64_t ws_limit_bytes(int dev) {
   int64_t v = g_ws_limit.load(std::memory_order_relaxed);
@@ -136,10 +136,10 @@ int64_t ws_limit_bytes(int dev) {
   return d;
 }
 
-// Returns with g_ws_mutex held when it succeeds; ws_release drops it.
+// Returns with the device's mutex held when it succeeds; ws_release drops it.
 hipError_t ws_acquire(int dev, size_t need, hipStream_t stream, void** out) {
-  g_ws_mutex.lock();
   Workspace& w = g_ws[dev];
+  w.mutex.lock();
   hipError_t e = hipSuccess;
   if (w.bytes < need || w.done == nullptr) {
     int cur = -1;
@@ -150,16 +150,21 @@ hipError_t ws_acquire(int dev, size_t need, hipStream_t stream, void** out) {
       // (hipFree waits for the device: nothing uses the old buffer any more)
       if (w.ptr != nullptr) (void)hipFree(w.ptr);
       w.ptr = nullptr; w.bytes = 0; w.used = false;
-      const size_t grow = need + need / 8;
+      size_t grow = need + need / 8;
       e = hipMalloc(&w.ptr, grow);
+      if (e != hipSuccess) {      // no room for the margin: exactly what this call needs
+        (void)hipGetLastError();
+        grow = need;
+        e = hipMalloc(&w.ptr, grow);
+      }
       if (e == hipSuccess) w.bytes = grow; else w.ptr = nullptr;
     }
     if (cur >= 0 && cur != dev) (void)hipSetDevice(cur);
   }
-  if (e == hipSuccess && w.used && w.last != stream) e = hipStreamWaitEvent(stream, w.done, 0);
+  if (e == hipSuccess && w.used) e = hipStreamWaitEvent(stream, w.done, 0);
   if (e != hipSuccess) {
     (void)hipGetLastError();
-    g_ws_mutex.unlock();
+    w.mutex.unlock();
     return e;
   }
   *out = w.ptr;
@@ -169,7 +174,6 @@ hipError_t ws_acquire(int dev, size_t need, hipStream_t stream, void** out) {
 void ws_release(int dev, hipStream_t stream) {
   Workspace& w = g_ws[dev];
   if (hipEventRecord(w.done, stream) == hipSuccess) {
-    w.last = stream;
     w.used = true;
   } else {
     // without the event the next call cannot order itself behind this one
@@ -177,7 +181,7 @@ void ws_release(int dev, hipStream_t stream) {
     (void)hipStreamSynchronize(stream);
     w.used = false;
   }
-  g_ws_mutex.unlock();
+  w.mutex.unlock();
 }
 
 // A call that holds the workspace (the repacking layer below) hands a part of it to the call it
@@ -1139,14 +1143,15 @@ int fa_v2_attn_bwd_compact_varlen(const fa_tensor4* q, const fa_tensor4* k, cons
 void fa_set_bwd_workspace_limit(int64_t bytes) { g_ws_limit.store(bytes, std::memory_order_relaxed); }
 
 int fa_trim_workspace(void) {
-  std::lock_guard<std::mutex> lock(g_ws_mutex);
   hipError_t err = hipSuccess;
-  for (int d = 0; d < kMaxDevices; ++d)
+  for (int d = 0; d < kMaxDevices; ++d) {
+    std::lock_guard<std::mutex> lock(g_ws[d].mutex);
     if (g_ws[d].ptr != nullptr) {
       const hipError_t e = hipFree(g_ws[d].ptr);      // waits for the device first
       g_ws[d].ptr = nullptr; g_ws[d].bytes = 0; g_ws[d].used = false;
       if (err == hipSuccess) err = e;
     }
+  }
   return (int)err;
 }
 
