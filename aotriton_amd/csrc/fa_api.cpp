@@ -456,13 +456,15 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   }
   int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2
-  if (be == 1 && (!is_16bit(dt) || s.d > 256 || s.elementwise)) {
-    // the vector-ALU kernels (fp32, head dims above 256, element-wise rows) exist for the split backend only: a forced fused backend cannot take the input, an
-    // unforced choice falls back to split when a delta buffer is there (template/op.cc:57-70)
+  if (be == 1 && (!is_16bit(dt) || s.d > 256)) {
+    // fp32 tensors and head dims above 256 have the split backend only: a forced fused backend cannot take the
+    // input, an unforced choice falls back to split when a delta buffer is there (template/op.cc:57-70)
     const bool forced = opt != nullptr && opt->force_backend_index >= 0;
     if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
     be = 0;
   }
+  // (the fused backend on tensors whose rows are not aligned 16-byte pieces runs on packed copies; whether
+  // the call gets the workspace for them is known at launch: fused_without_copies below)
   if (be == 0) {
     if (p->D.eager.ptr == nullptr && p->D.acquire == nullptr) return FA_ERROR_INVALID_VALUE;
     if (p->D.eager.ptr != nullptr && (e = check_row_stats(p->D.eager, s.row_stats)) != FA_SUCCESS) return e;
@@ -877,6 +879,13 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       ws_release(device_index(dev), stream);
       return rc;
     }
+  }
+  if (s.elementwise && backend == 1) {
+    // fused_without_copies: the element-wise kernels have the split backend only (same rule as in validate_bwd)
+    const bool forced = options != nullptr && options->force_backend_index >= 0;
+    if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
+    if (p->D.eager.ptr != nullptr && (e = check_row_stats(p->D.eager, s.row_stats)) != FA_SUCCESS) return e;
+    backend = 0;
   }
 
   fa::BwdArgs a{};

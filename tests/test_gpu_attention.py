@@ -197,6 +197,25 @@ def test_fp32_has_no_fused_backend():
         o.backward(do)
 
 
+@pytest.mark.parametrize('D,dtype', [(113, torch.bfloat16), (71, torch.float16)])
+def test_fused_backend_on_a_head_dim_that_is_no_multiple_of_8(D, dtype):
+    """The reference's fused backward takes any head dim (modules/flash/csrc/attn_bwd.cc:55-160 with the padding
+    of attn_fwd.cc:76-82).  Here it runs on packed copies; a call without workspace is refused when the backend
+    is forced (the element-wise kernels have the split backend only)."""
+    from aotriton_amd.autograd import attention, AttentionExtraArgs
+    from aotriton_amd._lib import lib
+    _run_case(2, 4, 2, 150, 131, D, dtype, True, dropout_p=0.1, bwd_backend=1, seed=D)
+    lib.fa_set_bwd_workspace_limit(0)
+    try:
+        q, k, v, _, do = make_inputs(1, 2, 2, 64, 64, D, dtype, DEV)
+        qg = q.clone().requires_grad_()
+        o, _, _ = attention(qg, k, v, None, False, 0.125, 0.0, AttentionExtraArgs(bwd_backend=1))
+        with pytest.raises(NotImplementedError):
+            o.backward(do)
+    finally:
+        lib.fa_set_bwd_workspace_limit(-1)
+
+
 def _sampled_grid_cases(n=72, seed=2024):
     """A seeded sample of the reference's test grids (tests/test_backward.py:35-142 with the
     lists of tests/_core_test_backward.py:60-89): regular, matrix bias, GQA, irregular
