@@ -184,6 +184,60 @@ def test_growing_shrinking_and_trimmed_workspace_on_two_streams():
                 assert (x.float() - y.float()).abs().max().item() <= tol, f'{name}, shape {shapes[i]}, round {rep}'
 
 
+def test_two_host_threads_share_the_workspace():
+    """Two host threads enqueue backwards of different sizes on a stream each, without synchronising
+    between calls: the calls take turns on the one buffer (mutex on the host, event on the GPU) and
+    every result equals the recomputing backward's within the rounding of delta."""
+    import threading
+    from aotriton_amd import flash
+    lib = _lib()
+    ok = flash.hipError_t.hipSuccess
+    shapes = [(1, 4, 2, 1024, 1024), (2, 2, 2, 384, 640)]
+    sm = 1.0 / math.sqrt(128)
+    jobs = []
+    for i, (B, Hq, Hk, Sq, Sk) in enumerate(shapes):
+        q, k, v, _, do = make_inputs(B, Hq, Hk, Sq, Sk, 128, torch.bfloat16, DEV, seed=40 + i)
+        o, L, dq, dk, dv, _ = _backward(q, k, v, None, do, sm, True, 0.0, 0)
+        jobs.append((q, k, v, do, o, L, (dq, dk, dv)))
+    lib.fa_set_bwd_workspace_limit(BIG)
+    assert lib.fa_trim_workspace() == 0          # the first calls of both threads race for the allocation
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    results, errors = {}, []
+
+    def worker(i):
+        try:
+            q, k, v, do, o, L, _ = jobs[i]
+            stream = torch.cuda.Stream()
+            outs = []
+            with torch.cuda.stream(stream):
+                for rep in range(6):
+                    dq, dk, dv = torch.full_like(q, float('nan')), torch.full_like(k, float('nan')), torch.full_like(v, float('nan'))
+                    delta = torch.empty_like(L)
+                    ext = flash.attn_options()
+                    ext.force_backend_index = 0
+                    assert flash.attn_bwd(q, k, v, None, sm, o, do, dq, dk, dv, None, None, L, delta, 0.0, null, null, 0,
+                                          True, extargs=ext) == ok
+                    outs.append((dq, dk, dv))
+            stream.synchronize()
+            results[i] = outs
+        except Exception as e:      # surfaces in the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(jobs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for i, outs in results.items():
+        want = jobs[i][6]
+        for rep, got in enumerate(outs):
+            for name, x, y in zip(('dq', 'dk', 'dv'), got, want):
+                tol = 2.0 ** -6 * y.float().abs().max().item()
+                assert (x.float() - y.float()).abs().max().item() <= tol, f'{name}, thread {i}, call {rep}'
+
+
 def test_headline_size_with_kept_ds():
     """B4 H32 S4096 D128 bf16 causal, the benchmark's shape, needs 4.3 GB of dS tiles: sampled heads
     against the recomputing kernels, and the closed forms that hold at any size (the first query sees
