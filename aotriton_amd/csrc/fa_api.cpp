@@ -279,6 +279,16 @@ int check_row_stats(const fa_tensor2& t, int64_t need) {
   return FA_SUCCESS;
 }
 
+// a contiguous fp32 (1, n) view for delta
+fa_tensor2 row_stats_view(void* ptr, int64_t n) {
+  fa_tensor2 t{};
+  t.ptr = ptr;
+  t.sizes[0] = 1; t.sizes[1] = (uint64_t)n;
+  t.strides[0] = (uint64_t)n; t.strides[1] = 1;
+  t.dtype = FA_DTYPE_FLOAT32;
+  return t;
+}
+
 fa::Strides3 strides3(const fa_tensor4& t) {
   return fa::Strides3{(int64_t)t.strides[0], (int64_t)t.strides[1], (int64_t)t.strides[2]};
 }
@@ -287,6 +297,7 @@ struct Shape {
   int batch, hq, hk, d, d_qk, d_v, max_sq, max_sk, num_seqlens;  // d: compiled head dim; d_qk, d_v: the tensors'; num_seqlens signed as in attn_fwd.cc:99
   bool windowed, bias, dropout;
   bool elementwise;       // some activation tensor is not made of aligned 16-byte pieces
+  bool fused_as_split;    // backend 1 asked for where no single-launch kernel exists (fp32, head dims above 256)
   int64_t row_stats;      // elements of L and of delta
 };
 
@@ -456,13 +467,12 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
   }
   int be = bwd_backend(p, opt);
   if (be < 0 || be > 1) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;   // e.g. the assembly backend 2
-  if (be == 1 && (!is_16bit(dt) || s.d > 256)) {
-    // fp32 tensors and head dims above 256 have the split backend only: a forced fused backend cannot take the
-    // input, an unforced choice falls back to split when a delta buffer is there (template/op.cc:57-70)
-    const bool forced = opt != nullptr && opt->force_backend_index >= 0;
-    if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
-    be = 0;
-  }
+  // fp32 tensors and head dims above 256 have no single-launch kernel: backend 1 runs the split kernels
+  // for them, with the caller's delta buffer when there is one and with one in the library's workspace
+  // otherwise (whether the call gets that is known at launch: attn_bwd_impl)
+  s.fused_as_split = be == 1 && (!is_16bit(dt) || s.d > 256);
+  if (s.fused_as_split && p->D.eager.ptr != nullptr && (e = check_row_stats(p->D.eager, s.row_stats)) != FA_SUCCESS)
+    return e;
   // (the fused backend on tensors whose rows are not aligned 16-byte pieces runs on packed copies; whether
   // the call gets the workspace for them is known at launch: fused_without_copies below)
   if (be == 0) {
@@ -846,7 +856,10 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     // packed copies of the eight activation tensors, the MFMA kernels on those, dQ, dK, dV copied back;
     // the packed call gets the rest of the buffer for its own use (dS)
     const fa_tensor4* all[8] = {&p->Q, &p->K, &p->V, &p->Out, &p->DO, &p->DQ, &p->DK, &p->DV};
-    const size_t copies = bwd_copies_bytes(p);
+    // (a call for backend 1 that will run the split kernels and brings no delta buffer gets one here)
+    const bool lib_delta = backend == 1 && s.fused_as_split && p->D.eager.ptr == nullptr && p->D.acquire == nullptr;
+    const size_t delta_bytes = lib_delta ? (((size_t)s.row_stats * 4 + 255) & ~(size_t)255) : 0;
+    const size_t copies = bwd_copies_bytes(p) + delta_bytes;
     fa_bwd_params p2 = *p;
     fa_tensor4* to[8] = {&p2.Q, &p2.K, &p2.V, &p2.Out, &p2.DO, &p2.DQ, &p2.DK, &p2.DV};
     for (int i = 0; i < 8; ++i) *to[i] = packed_view(*all[i], reinterpret_cast<void*>(uintptr_t(256)));   // shapes first
@@ -869,6 +882,11 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
         at += packed_bytes(*all[i]);
         if (i < 5 && err == hipSuccess) err = repack(*all[i], *to[i], false, stream);
       }
+      if (lib_delta) {
+        p2.D = fa_lazy_tensor2{};
+        p2.D.eager = row_stats_view(at, s.row_stats);
+        at += delta_bytes;
+      }
       int rc = (int)err;
       if (err == hipSuccess) {
         t_ws_nested = NestedWorkspace{true, inner > 0 ? at : nullptr, (size_t)inner};
@@ -880,8 +898,32 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       return rc;
     }
   }
+  if (backend == 1 && s.fused_as_split) {
+    // the split kernels: with the caller's delta buffer, or with one in the workspace
+    if (kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;      // there is no such kernel to run alone
+    if (p->D.eager.ptr != nullptr || p->D.acquire != nullptr) {
+      backend = 0;
+    } else {
+      const size_t bytes = ((size_t)s.row_stats * 4 + 255) & ~(size_t)255;
+      void* base = nullptr;
+      if (kernel_slot >= 0 || t_ws_nested.active || stream_is_capturing(stream) ||
+          (int64_t)bytes > ws_limit_bytes(device_index(dev)) ||
+          ws_acquire(device_index(dev), bytes, stream, &base) != hipSuccess)
+        return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
+      fa_bwd_params p2 = *p;
+      p2.D = fa_lazy_tensor2{};
+      p2.D.eager = row_stats_view(base, s.row_stats);
+      fa_options split = options != nullptr ? *options : fa_options{};
+      split.force_backend_index = 0;
+      t_ws_nested = NestedWorkspace{true, nullptr, 0};
+      const int rc = attn_bwd_impl(&p2, params_version, hip_stream, &split, -1, false);
+      t_ws_nested = NestedWorkspace{};
+      ws_release(device_index(dev), stream);
+      return rc;
+    }
+  }
   if (s.elementwise && backend == 1) {
-    // fused_without_copies: the element-wise kernels have the split backend only (same rule as in validate_bwd)
+    // fused_without_copies: the element-wise kernels have the split backend only
     const bool forced = options != nullptr && options->force_backend_index >= 0;
     if (forced || (p->D.eager.ptr == nullptr && p->D.acquire == nullptr)) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
     if (p->D.eager.ptr != nullptr && (e = check_row_stats(p->D.eager, s.row_stats)) != FA_SUCCESS) return e;

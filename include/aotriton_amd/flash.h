@@ -231,8 +231,13 @@ FA_API int fa_attn_fwd(const fa_fwd_params* params, int32_t params_version,
 
 /* v3::flash::attn_bwd -- include/aotriton/flash.h:176-180,
  * modules/flash/csrc/attn_bwd.cc:55-160.
- * Same tensors as the forward.  fp32 tensors, head dims above 256 and the element-wise kernels have
- * the split backend only.  DB with packed tokens is rejected (FA_ERROR_NOT_SUPPORTED): all sequences
+ * Same tensors as the forward.  Single-launch kernels (backend 1) exist for fp16/bf16 up to head dim
+ * 256.  For fp32 tensors and head dims above 256 backend 1 runs the split kernels: with params->D when
+ * the caller brings one, else with delta in the library's workspace; tensors whose rows are not aligned
+ * 16-byte pieces reach either backend through packed copies in the workspace.  A call for backend 1
+ * that would need the workspace and cannot have it (limit, stream capture) answers
+ * FA_ERROR_PEER_ACCESS_UNSUPPORTED when the backend is forced or no delta buffer is there, and runs the
+ * split backend otherwise.  DB with packed tokens is rejected (FA_ERROR_NOT_SUPPORTED): all sequences
  * share one bias there. */
 FA_API int fa_attn_bwd(const fa_bwd_params* params, int32_t params_version,
                        void* hip_stream, const fa_options* options);

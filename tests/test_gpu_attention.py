@@ -188,13 +188,40 @@ def test_head_dim_512_with_bias_and_dropout():
     _run_case(1, 2, 2, 100, 100, 512, torch.bfloat16, True, dropout_p=0.2, bias=True, bwd_backend=0)
 
 
-def test_fp32_has_no_fused_backend():
-    from aotriton_amd.autograd import attention, AttentionExtraArgs
-    q, k, v, _, do = make_inputs(1, 2, 2, 64, 64, 64, torch.float32, DEV)
-    qg = q.clone().requires_grad_()
-    o, _, _ = attention(qg, k, v, None, False, 0.125, 0.0, AttentionExtraArgs(bwd_backend=1))
-    with pytest.raises(NotImplementedError):      # hipErrorPeerAccessUnsupported: the backend cannot take the input
-        o.backward(do)
+@pytest.mark.parametrize('dtype,D', [(torch.float32, 64), (torch.bfloat16, 512), (torch.float32, 300)])
+def test_backend_1_where_no_single_launch_kernel_exists(dtype, D):
+    """The reference compiles its fused backward for fp32 too (modules/flash/aot/bwd_kernel_fuse.py:25-28).
+    Here fp32 tensors and head dims above 256 have split kernels only; a call for backend 1, which brings
+    no delta buffer (v2 attn_bwd_fused), runs them with delta in the library's workspace: same results as
+    backend 0, bit for bit.  Without workspace the call is refused."""
+    from aotriton_amd import flash
+    from aotriton_amd._lib import lib
+    ok = flash.hipError_t.hipSuccess
+    B, H, Sq, Sk = 2, 2, 100, 77
+    q, k, v, _, do = make_inputs(B, H, H, Sq, Sk, D, dtype, DEV, seed=3)
+    sm = D ** -0.5
+    null = torch.empty([0], device=DEV, dtype=torch.uint64)
+    atomic = torch.zeros([1], device=DEV, dtype=torch.int32)
+    o = torch.empty_like(q)
+    L = torch.empty(B * H, Sq, device=DEV, dtype=torch.float32)
+    assert flash.attn_fwd(q, k, v, None, sm, L, o, 0.0, null, null, 0, null, null, None, True, atomic) == ok
+    want = [torch.empty_like(t) for t in (q, k, v)]
+    delta = torch.empty_like(L)
+    ext = flash.attn_options()
+    ext.force_backend_index = 0
+    assert flash.attn_bwd(q, k, v, None, sm, o, do, *want, None, None, L, delta, 0.0, null, null, 0, True,
+                          extargs=ext) == ok
+    got = [torch.full_like(t, float('nan')) for t in (q, k, v)]
+    assert flash.attn_bwd_fused(q, k, v, None, sm, o, do, *got, None, L, 0.0, null, null, 0, True) == ok
+    torch.cuda.synchronize()
+    for name, x, y in zip(('dq', 'dk', 'dv'), got, want):
+        assert torch.equal(x, y), name
+    lib.fa_set_bwd_workspace_limit(0)
+    try:
+        assert flash.attn_bwd_fused(q, k, v, None, sm, o, do, *got, None, L, 0.0, null, null, 0, True) == \
+            flash.hipError_t.hipErrorPeerAccessUnsupported
+    finally:
+        lib.fa_set_bwd_workspace_limit(-1)
 
 
 @pytest.mark.parametrize('D,dtype', [(113, torch.bfloat16), (71, torch.float16)])
@@ -501,8 +528,6 @@ def test_empty_tensors(shape, backend, dtype):
     # no batch element, no query row, no key: the calls succeed; without a key O = 0,
     # LSE = +inf and dQ = 0; without a query dK = dV = 0
     from aotriton_amd.autograd import attention, AttentionExtraArgs
-    if dtype == torch.float32 and backend == 1:
-        pytest.skip('fp32 has the split backend only')
     B, Sq, Sk = shape
     H, D = 2, 64
     q = torch.randn(B, H, Sq, D, device=DEV).to(dtype).requires_grad_()

@@ -114,8 +114,6 @@ def _run_varlen_case(lq, lk, Hq, Hk, D, dtype, causal, backend, p=0.0, seed=11):
 def test_compact_varlen_with_empty_sequences(dtype, causal, backend):
     # sequences without queries, without keys and without both among ordinary ones, and
     # query and key lengths that differ
-    if dtype == torch.float32 and backend == 1:
-        pytest.skip('fp32 has the split backend only')
     _run_varlen_case([5, 0, 70, 0, 33, 130], [9, 64, 0, 0, 33, 40], 4, 2, 64, dtype, causal, backend)
 
 
@@ -500,8 +498,6 @@ def test_varlen_with_bias(layout, dtype, D, backend):
     tokens (no dB then).  Against the oracle, sequence by sequence."""
     from aotriton_amd import flash
     from oracle import fa_ref
-    if dtype == torch.float32 and backend == 1:
-        pytest.skip('fp32 has the split backend only')
     lens = np.asarray([70, 5, 0, 131, 64])
     n, mx, Hq, Hk = len(lens), int(lens.max()), 4, 2
     g = torch.Generator().manual_seed(21)
