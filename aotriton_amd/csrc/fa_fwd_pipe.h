@@ -326,7 +326,11 @@ __device__ __forceinline__ void fwd_item_pipe(const FwdArgs& a, const int z, con
         for (int i = 0; i < 16; ++i) x[qb][i] *= qk_scale;
       }
       if (kBias) {
-        if (bias_vec && (u + 1) * 32 <= si.seqlen_k) {
+        if (bias_co && u <= u1 && (u + 1) * 32 <= si.seqlen_k) {
+          // the unit's pieces were fetched a step ago and handed over in the layout of S^T (fetch_bias, hand_over)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) x[qb][i] += (float)bin[qb][i / 4][i % 4] * kLog2e;   // fwd_kernel_inner.py:187
+        } else if (bias_vec && (u + 1) * 32 <= si.seqlen_k) {
           // a lane's four consecutive keys of every 8-key group in one 8-byte load
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
