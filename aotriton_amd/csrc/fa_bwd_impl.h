@@ -462,6 +462,10 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     }
   };
 
+  // seed and offset of the dropout mask: read once per item, not once per tile
+  DropoutState drop0{};
+  if (kDropout) drop0 = make_dropout_base(a.drop, a.seq.max_seqlen_k);
+
   // ---- one (q-head, Q tile) step -----------------------------------------------
   auto compute = [&](auto masked_tag, int g, int e, int stage, bool live, int g_nxt, int e_nxt) {
     constexpr bool masked = decltype(masked_tag)::value;
@@ -483,7 +487,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     DropoutState dst{};
-    if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
+    if (kDropout) dst = dropout_for_head(drop0, z, hq, a.hq, a.seq.max_seqlen_q);
     if constexpr (kStoreDs) {
       // (the tiles of a q-head follow each other)
       ds_tile = e == 0 ? reinterpret_cast<char*>(a.ds_ws) +

@@ -508,6 +508,9 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
     fetch(0);
     publish();
     __syncthreads();
+    // seed and offset of the dropout mask: read once, not once per tile
+    DropoutState drop0{};
+    if (kDropout) drop0 = make_dropout_base(a.drop, a.seq.max_seqlen_k);
     for (int it = 0; it < total; ++it) {
       const int hq = hk * group + it / ntq;
       const int e = br.lo + it % ntq;
@@ -530,7 +533,7 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_d512_kernel(const BwdArgs a) {
       const f32x4 dp4 = part_sum_quarter(partD, wave, lane);
 
       DropoutState dst{};
-      if (kDropout) dst = make_dropout(a.drop, z, hq, a.hq, a.seq.max_seqlen_q, a.seq.max_seqlen_k);
+      if (kDropout) dst = dropout_for_head(drop0, z, hq, a.hq, a.seq.max_seqlen_q);
       const T* bptr = nullptr;
       if (kBias)
         bptr = reinterpret_cast<const T*>(a.bias) + (int64_t)si.batch_index * a.sb_z + (int64_t)hq * a.sb_h +

@@ -217,21 +217,35 @@ struct DropoutState {
   float scale;       // 1/(1-p)
 };
 
-__device__ __forceinline__ DropoutState make_dropout(const DropoutArgs& d, int z, int h, int hq,
-                                                     int max_seqlen_q, int max_seqlen_k) {
+// The part that reads memory (seed and offset are device scalars): once per work item.  A kernel
+// that walks several heads keeps this and calls dropout_for_head per head; reading the two scalars
+// again for every tile costs two L2 round trips that nothing hides.
+__device__ __forceinline__ DropoutState make_dropout_base(const DropoutArgs& d, int max_seqlen_k) {
   DropoutState s;
   const uint64_t seed = d.seed_ptr ? *d.seed_ptr : 0ull;
   uint64_t base = d.offset2;
   if (d.offset1_ptr) base += *d.offset1_ptr;
   s.k0 = (uint32_t)seed; s.k1 = (uint32_t)(seed >> 32);
   s.stride = (uint32_t)((max_seqlen_k + 3) / 4);
-  // modules/flash/kernel/fwd_kernel.py:405-407: the per-head term is a product of int32
-  // values there, so it wraps modulo 2^32 and is sign-extended into the 64-bit base.
-  const uint32_t head_term = (uint32_t)(z * hq + h) * (uint32_t)max_seqlen_q * s.stride;
-  s.base = base + (uint64_t)(int64_t)(int32_t)head_term;
+  s.base = base;
   s.thr = dropout_threshold(d.p);
   s.scale = 1.0f / (1.0f - d.p);
   return s;
+}
+
+__device__ __forceinline__ DropoutState dropout_for_head(const DropoutState& s0, int z, int h, int hq,
+                                                         int max_seqlen_q) {
+  DropoutState s = s0;
+  // modules/flash/kernel/fwd_kernel.py:405-407: the per-head term is a product of int32
+  // values there, so it wraps modulo 2^32 and is sign-extended into the 64-bit base.
+  const uint32_t head_term = (uint32_t)(z * hq + h) * (uint32_t)max_seqlen_q * s.stride;
+  s.base = s0.base + (uint64_t)(int64_t)(int32_t)head_term;
+  return s;
+}
+
+__device__ __forceinline__ DropoutState make_dropout(const DropoutArgs& d, int z, int h, int hq,
+                                                     int max_seqlen_q, int max_seqlen_k) {
+  return dropout_for_head(make_dropout_base(d, max_seqlen_k), z, h, hq, max_seqlen_q);
 }
 
 // Keep bits of columns n0..n0+3 (n0 % 4 == 0) of row m, bit r <-> column n0+r.
