@@ -12,8 +12,11 @@
  *   - philox seed/offset and the persistent counter are DEVICE pointers
  *     (include/aotriton/flash.h:113-120);
  *   - launches are asynchronous on the caller's stream, nothing is synchronised;
- *   - the library never allocates device memory, except through the caller's
- *     lazy-tensor callbacks (include/aotriton/util.h:224-246).
+ *   - device memory comes from the caller, directly or through its lazy-tensor
+ *     callbacks (include/aotriton/util.h:224-246).
+ * One departure from the last point: the library keeps one workspace buffer per device
+ * (fa_set_bwd_workspace_limit below: what it is for, how it is bounded, how to switch it
+ * off).  Calls on a stream under capture and fa_attn_bwd_noalloc never touch it.
  */
 #ifndef AOTRITON_AMD_FLASH_H
 #define AOTRITON_AMD_FLASH_H
