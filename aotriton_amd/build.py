@@ -52,6 +52,7 @@ def sources():
 def headers():
     hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith('.h')]
     hs.append(os.path.join(ROOT, 'include', 'aotriton_amd', 'flash.h'))
+    hs.append(os.path.join(ROOT, 'include', 'aotriton_amd', 'probe.h'))
     return hs
 
 

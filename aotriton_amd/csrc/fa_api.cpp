@@ -13,6 +13,7 @@
 #include <mutex>
 
 #include "aotriton_amd/flash.h"
+#include "aotriton_amd/probe.h"
 #include "fa_args.h"
 #include "fa_intervals.h"
 #include "fa_kernels.h"

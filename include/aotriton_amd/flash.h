@@ -379,14 +379,6 @@ FA_API int fa_get_multiprocessor_count(void* hip_stream);
  * reference's timing method; it reads the device properties the same way). */
 FA_API int fa_get_clock_rate_khz(void* hip_stream);
 
-/* Benchmark aid without a counterpart in the reference: a register-only loop of
- * v_mfma_f32_32x32x16_bf16 (num_workgroups x 4 waves x iters x 32 MFMAs), on constant operands
- * or on operands with random mantissas.  out: num_workgroups * 256 floats (device);
- * clocks: 2 x uint64 (device) = shader cycles and 100 MHz reference ticks of workgroup 0.
- * Timed by the caller; FLOP per launch = num_workgroups * 4 * iters * 32 * 32768. */
-FA_API int fa_probe_mfma_rate(int32_t random_operands, int32_t num_workgroups, int32_t iters,
-                              float* out, uint64_t* clocks, void* hip_stream);
-
 /* bindings/hipruntime.cc:11-95 */
 FA_API int fa_hip_get_last_error(void);
 FA_API int fa_hip_device_synchronize(void);

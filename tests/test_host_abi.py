@@ -22,7 +22,8 @@ def _lib():
 
 def test_exports_every_declared_symbol():
     L = _lib()
-    hdr = open(os.path.join(ROOT, 'include', 'aotriton_amd', 'flash.h')).read()
+    import glob
+    hdr = '\n'.join(open(h).read() for h in sorted(glob.glob(os.path.join(ROOT, 'include', 'aotriton_amd', '*.h'))))
     declared = set(re.findall(r'FA_API\s+[\w\s\*]+?\b(fa_\w+)\s*\(', hdr))
     assert declared, 'no declarations parsed'
     assert declared == set(L.SYMBOLS), (declared ^ set(L.SYMBOLS))
