@@ -239,6 +239,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
   op_t sb[TS];                         // dS operands of the dK GEMM; with kStoreDs they outlive their tile
   char* ds_tile = nullptr;             // stored tile of the running (q-head, Q tile) step
   constexpr int kDsSlots = 4;
+  // cache policy bits of the stores: non-temporal (the tile is read once, by another kernel) at agent scope;
+  // measured against the other combinations of sc0 / sc1 / nt on one box: 1-2 % of the kernel
+  constexpr int kDsStorePolicy = 2 | 16;
   auto ds_slot_of = [](int t) { return TS >= kDsSlots ? t * kDsSlots / TS : 2 * t + 1; };
   auto store_ds_slot = [&](char* tile, int slot) {
     if constexpr (kStoreDs) {
@@ -247,7 +250,7 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       for (int t = 0; t < TS; ++t)
         if (ds_slot_of(t) == slot)
           __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, sb[t]), rs, ds_pos[t & 1],
-                                                 DT::piece(0, t) + wave_u * 2048, 2);
+                                                 DT::piece(0, t) + wave_u * 2048, kDsStorePolicy);
     }
   };
 
