@@ -46,7 +46,8 @@ __global__ void bwd_preprocess_kernel(const BwdArgs a) {
   if (row < si.seqlen_q && cc * 8 < a.head_dim_v) {   // columns past the head dim of Out and dOut do not exist
     const int64_t ro = (int64_t)si.batch_index * a.so.z + (int64_t)h * a.so.h + (int64_t)(si.q_start + row) * a.so.s;
     const int64_t rd = (int64_t)si.batch_index * a.sdo.z + (int64_t)h * a.sdo.h + (int64_t)(si.q_start + row) * a.sdo.s;
-    const op_t o = *reinterpret_cast<const op_t*>(reinterpret_cast<const T*>(a.out) + ro + cc * 8);
+    // (O is read here and nowhere else in the backward: a streaming load; dO stays cached for the dK/dV kernel)
+    const op_t o = __builtin_nontemporal_load(reinterpret_cast<const op_t*>(reinterpret_cast<const T*>(a.out) + ro + cc * 8));
     const op_t d = *reinterpret_cast<const op_t*>(reinterpret_cast<const T*>(a.dout) + rd + cc * 8);
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc += (float)o[e] * (float)d[e];
