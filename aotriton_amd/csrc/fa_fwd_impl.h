@@ -182,7 +182,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
     op_t qin[32 / RPQ];
 #pragma unroll
     for (int i = 0; i < 32 / RPQ; ++i)
-      qin[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(qrs, qvoff, i * RPQ * (int)a.sq.s * 2, 0));
+      qin[i] = __builtin_bit_cast(op_t, __builtin_amdgcn_raw_buffer_load_b128(qrs, qvoff, i * RPQ * (int)a.sq.s * 2, 2));
 #pragma unroll
     for (int i = 0; i < 32 / RPQ; ++i)
       *reinterpret_cast<op_t*>(rowbuf + (i * RPQ + rq) * SM::ROW_STR + cq * 16) = qin[i];
@@ -540,7 +540,7 @@ __device__ __forceinline__ void fwd_item(const FwdArgs& a, const int z, const in
 #pragma unroll
     for (int i = 0; i < 32 / RPQ; ++i) {
       const op_t x = *reinterpret_cast<const op_t*>(rowbuf + (i * RPQ + rq) * SM::ROW_STR + cq * 16);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), ors, ovoff, i * RPQ * (int)a.so.s * 2, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), ors, ovoff, i * RPQ * (int)a.so.s * 2, 2);
     }
   }
   if (row_ok && lse_ptr && hi == 0)
