@@ -262,6 +262,33 @@ def test_headline_size_with_kept_ds():
     assert a[2][:, :, 0].float().abs().max().item() <= 1e-2
 
 
+def test_no_room_for_the_workspace_means_recomputing():
+    """When hipMalloc cannot deliver the workspace (the caller's allocator holds the device's memory) the
+    call recomputes instead of failing: same results as with the limit at 0, bit for bit."""
+    B, H, S, D = 4, 32, 4096, 128                      # needs 4.4 GB of dS tiles
+    g = torch.Generator(device=DEV).manual_seed(99)
+    rn = lambda: torch.randn(B, H, S, D, device=DEV, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v, do = rn(), rn(), rn(), rn()
+    sm = 1.0 / math.sqrt(D)
+    want = _backward(q, k, v, None, do, sm, True, 0.0, 0)
+    assert _lib().fa_trim_workspace() == 0
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info()
+    if free < (16 << 30):
+        pytest.skip('not enough free device memory to stage the case')
+    try:
+        hog = torch.empty(free - (2 << 30), device=DEV, dtype=torch.int8)      # leaves 2 GiB
+    except RuntimeError:
+        pytest.skip('could not take the device memory in one piece')
+    try:
+        got = _backward(q, k, v, None, do, sm, True, 0.0, BIG)
+    finally:
+        del hog
+        torch.cuda.empty_cache()
+    for name, x, y in zip(('dq', 'dk', 'dv'), got[2:5], want[2:5]):
+        assert torch.equal(x, y), name
+
+
 def test_packed_copies_take_odd_head_dims_to_the_mfma_kernels():
     """Head dim 113 (one of the reference's, modules/flash/tests/test_forward.py:22): with workspace the
     queries report packed copies (bit 5), with the limit at 0 they do not; both give the oracle's results
