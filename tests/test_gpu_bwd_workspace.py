@@ -1,5 +1,5 @@
 """The split backward that keeps dS in HBM (dK/dV kernel writes it, a dQ = dS K kernel reads it
-back) against the oracle and against the recomputing kernels, through the C ABI.
+back; head dims 72 to 256) against the oracle and against the recomputing kernels, through the C ABI.
 
 The reference's split backward always recomputes S and dP in its dQ kernel
 (modules/flash/kernel/bwd_kernel_dq.py:45-389); both ways must give its results.  Tolerances are
@@ -84,6 +84,13 @@ CASES = [
     (1, 1, 1, 1, 1, 128, torch.bfloat16, True, 0.0, False, False),
     (1, 2, 2, 64, 2048, 128, torch.bfloat16, False, 0.0, False, False),
     (1, 2, 2, 2048, 64, 128, torch.bfloat16, True, 0.0, False, False),
+    # the 256-column build (32-query tiles)
+    (2, 4, 2, 300, 264, 256, torch.float16, True, 0.0, False, False),
+    (1, 3, 3, 523, 337, 256, torch.bfloat16, False, 0.0, False, True),
+    (1, 2, 1, 777, 1301, 256, torch.float16, (100, 20), 0.2, False, False),
+    (1, 2, 2, 333, 257, 192, torch.bfloat16, True, 0.1, True, False),
+    (2, 2, 1, 129, 65, 136, torch.float16, False, 0.0, False, False),
+    (1, 1, 1, 1, 1, 256, torch.bfloat16, True, 0.0, False, False),
 ]
 
 
@@ -124,13 +131,16 @@ def test_both_backwards_meet_the_oracle(case):
 
 
 def test_calls_that_do_not_qualify_recompute():
-    """head dims outside 72-128, fp32, packed sequences and dB keep the recomputing kernels"""
+    """head dims up to 64 (where keeping dS measured slower), fp32, packed sequences and dB keep the recomputing kernels"""
     from aotriton_amd import flash
     _lib().fa_set_bwd_workspace_limit(BIG)
     sm = 0.1
-    for D, dtype in ((64, torch.bfloat16), (256, torch.float16), (128, torch.float32), (40, torch.bfloat16)):
+    for D, dtype in ((64, torch.bfloat16), (128, torch.float32), (40, torch.bfloat16), (512, torch.bfloat16)):
         q, k, v, b, do = make_inputs(1, 2, 2, 128, 128, D, dtype, DEV, seed=1)
         assert not _would_keep_ds(q, k, v, None, do, sm, True, 0.0), (D, dtype)
+    for D in (72, 256):
+        q, k, v, b, do = make_inputs(1, 2, 2, 128, 128, D, torch.float16, DEV, seed=1)
+        assert _would_keep_ds(q, k, v, None, do, sm, True, 0.0), D
     q, k, v, b, do = make_inputs(1, 2, 2, 128, 128, 128, torch.bfloat16, DEV, seed=1)
     assert _would_keep_ds(q, k, v, None, do, sm, True, 0.0)
     # a limit below the need (2 bytes per (head, query, key) pair, in tiles of 128 x 64, plus the row statistics)
