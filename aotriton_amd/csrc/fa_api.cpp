@@ -513,9 +513,12 @@ fa::DropoutArgs dropout_args(float p, const fa_tensor0& seed, const fa_tensor0& 
 // packed sequences, dB wanted, an empty tensor).  *ds_bytes / *stat_bytes: the parts of the buffer.
 int64_t ds_workspace_need(const fa_bwd_params* p, const Shape& s, int* ntq, int* ntk, int64_t* ds_bytes,
                           int64_t* stat_bytes) {
-  if (s.elementwise || !is_16bit(p->Q.dtype) || (s.d != 128 && s.d != 256) || s.num_seqlens != 0 || p->DB.ptr != nullptr ||
+  if (s.elementwise || !is_16bit(p->Q.dtype) || (s.d != 64 && s.d != 128 && s.d != 256) || s.num_seqlens != 0 || p->DB.ptr != nullptr ||
       s.batch <= 0 || s.max_sq <= 0 || s.max_sk <= 0)
     return 0;
+  // the 64-column build: 2 bytes per pair are too many for its little GEMM work unless the dQ kernel is
+  // spared a bias or the Philox arithmetic (same box, stored / recomputing: 1.05-1.14 plain, 0.69-0.81 with either)
+  if (s.d == 64 && !s.dropout && !s.bias) return 0;
   int64_t tile_bytes = 0;
   fa::ds_tile_counts(p->Q.dtype, s.d, s.max_sq, s.max_sk, ntq, ntk, &tile_bytes);
   *ds_bytes = (int64_t)s.batch * s.hq * *ntq * *ntk * tile_bytes;

@@ -1560,8 +1560,8 @@ hipError_t launch_dkdv_variant(const BwdArgs& a0, hipStream_t stream) {
   // (the level table's LDS is requested whether or not this launch uses it: the kernel's limit is set once)
   constexpr int smem = DkDvSmem<D, BM>::BYTES + (D < 256 ? kLevelBytes : 0);
   if (a.ds_ws != nullptr) {
-    // (the variant that stores dS exists where it pays: the 128- and 256-column builds)
-    if constexpr (D == 128 || D == 256)
+    // (every build has the variant that stores dS; the host decides where it pays)
+    if constexpr (D == 64 || D == 128 || D == 256)
       return launch_with_lds<bwd_dkdv_kernel<T, D, NW, BM, W, B, P, kPad, true>>(grid, NW * 64, smem, stream, a);
     else
       return hipErrorNotSupported;

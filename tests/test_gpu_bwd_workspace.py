@@ -91,6 +91,11 @@ CASES = [
     (1, 2, 2, 333, 257, 192, torch.bfloat16, True, 0.1, True, False),
     (2, 2, 1, 129, 65, 136, torch.float16, False, 0.0, False, False),
     (1, 1, 1, 1, 1, 256, torch.bfloat16, True, 0.0, False, False),
+    # the 64-column build (128-query tiles): with dropout or a bias only
+    (2, 4, 2, 300, 264, 64, torch.float16, True, 0.2, False, False),
+    (1, 3, 3, 523, 337, 64, torch.bfloat16, False, 0.1, False, True),
+    (1, 2, 1, 777, 1301, 40, torch.float16, (100, 20), 0.3, False, False),
+    (1, 2, 2, 129, 257, 16, torch.bfloat16, True, 0.5, False, False),
 ]
 
 
@@ -131,7 +136,8 @@ def test_both_backwards_meet_the_oracle(case):
 
 
 def test_calls_that_do_not_qualify_recompute():
-    """head dims up to 64 (where keeping dS measured slower), fp32, packed sequences and dB keep the recomputing kernels"""
+    """head dims up to 64 without dropout and bias (where keeping dS measured slower), head dims above 256, fp32,
+    packed sequences and dB keep the recomputing kernels"""
     from aotriton_amd import flash
     _lib().fa_set_bwd_workspace_limit(BIG)
     sm = 0.1
@@ -141,6 +147,8 @@ def test_calls_that_do_not_qualify_recompute():
     for D in (72, 256):
         q, k, v, b, do = make_inputs(1, 2, 2, 128, 128, D, torch.float16, DEV, seed=1)
         assert _would_keep_ds(q, k, v, None, do, sm, True, 0.0), D
+    q, k, v, b, do = make_inputs(1, 2, 2, 128, 128, 64, torch.float16, DEV, seed=1)
+    assert _would_keep_ds(q, k, v, None, do, sm, True, 0.1)
     q, k, v, b, do = make_inputs(1, 2, 2, 128, 128, 128, torch.bfloat16, DEV, seed=1)
     assert _would_keep_ds(q, k, v, None, do, sm, True, 0.0)
     # a limit below the need (2 bytes per (head, query, key) pair, in tiles of 128 x 64, plus the row statistics)
