@@ -100,6 +100,8 @@ def main():
     ap.add_argument('--only', default=None, choices=['c4', 'c5'],
                     help='run only the forward and the backward of configuration 4 (packed sequences) or 5 (D=256, window + '
                          'bias + dropout) a few times and print their times (for profiler runs)')
+    ap.add_argument('--recompute', action='store_true',
+                    help='with --only: workspace limit 0, i.e. the backward whose dQ kernel recomputes S and dP')
     ap.add_argument('--mfma-peak', action='store_true',
                     help='only measure what the matrix pipe sustains (register-only MFMA loop, constant '
                          'and random operands) and print that as one JSON line')
@@ -212,6 +214,8 @@ def main():
     if args.only:
         null = torch.empty([0], device=dev, dtype=torch.uint64)
         atomic = torch.zeros([1], device=dev, dtype=torch.int32)
+        if args.recompute:
+            lib.fa_set_bwd_workspace_limit(0)
         f, b, fl, work = make_c4() if args.only == 'c4' else make_c5()
         runs = {'fwd': f, 'bwd': b} if args.only == 'c4' else {'fwd': f, 'bwd_no_db': lambda: b(False)}
         res = {}
