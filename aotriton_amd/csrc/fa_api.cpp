@@ -984,12 +984,12 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     // out; the dK/dV kernel runs after it and reads it, so the whole backward is two launches
     // (kernel_slot 0 still launches the preprocess kernel on its own).
     const bool delta_launch = f32 || big || slow;
-    // The 16-bit kernels at head dims 72-128 can keep dS in HBM instead of recomputing S and dP in
+    // The 16-bit kernels up to head dim 256 can keep dS in HBM instead of recomputing S and dP in
     // the dQ kernel (5 GEMMs instead of 7): delta first, then dK/dV writing dS, then dQ = dS K.  It
     // takes 2 bytes per (query, key) pair of workspace; when that is above the limit, under stream
-    // capture, for packed sequences or with dB the kernels recompute.  (Measured at B4 S4096, bf16
-    // causal: head dim 128 gains, head dim 64, where a pair costs half the arithmetic and the same
-    // bytes, loses 13 %.)
+    // capture, for packed sequences or with dB the kernels recompute.  (Measured at S4096, 16384 tokens:
+    // head dim 128 gains 5 %, 256 gains 16 %; head dim 64, where a pair costs half the arithmetic and
+    // the same bytes, loses 12 % unless the dQ kernel is spared dropout or a bias: then it gains 20-30 %.)
     void* ds_ws = nullptr;
     int ntq = 0, ntk = 0;
     int64_t ds_bytes = 0, stat_bytes = 0;

@@ -436,9 +436,17 @@ def main():
         torch.cuda.empty_cache()
         # --- configuration 5: B2 H16 S8192 D256 fp16, window (1024, 0) + bias + dropout 0.1 ----------
         fwd5, bwd5, fl5, work5 = make_c5()
+
+        def with_limit0(fn):
+            lib.fa_set_bwd_workspace_limit(0)
+            fn()
+            lib.fa_set_bwd_workspace_limit(-1)
+
         out['c5'] = {'workload': work5,
                      'fwd': row(fl5, do_bench(fwd5, max_reps=100)),
                      'bwd_split_no_db': row(2.5 * fl5, do_bench(lambda: bwd5(False), max_reps=60)),
+                     'bwd_split_no_db_recompute': row(2.5 * fl5, do_bench(lambda: with_limit0(lambda: bwd5(False)), max_reps=60),
+                                                      {'note': 'workspace limit 0: the dQ kernel recomputes S and dP, with bias and dropout'}),
                      'bwd_split_with_db': row(2.5 * fl5, do_bench(lambda: bwd5(True), max_reps=60),
                                               {'note': 'dB is a dense (B,H,S,S) tensor: 4 GiB written, zeros outside the band'})}
         del fwd5, bwd5

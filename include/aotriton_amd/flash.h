@@ -305,8 +305,8 @@ FA_API int fa_v2_attn_bwd_compact_varlen(
 FA_API int fa_attn_bwd_noalloc(const fa_bwd_params* params, int32_t params_version,
                                void* hip_stream);
 
-/* Workspace of the split backward.  For 16-bit tensors at head dims 72-128 (dense batches, no dB,
- * not under stream capture) fa_attn_bwd keeps dS in HBM between its dK/dV and dQ kernels instead of
+/* Workspace of the split backward.  For 16-bit tensors at head dims up to 256 (dense batches, no dB,
+ * not under stream capture; up to head dim 64 only with dropout or a bias, where it pays) fa_attn_bwd keeps dS in HBM between its dK/dV and dQ kernels instead of
  * recomputing S and dP in the dQ kernel (5 GEMMs instead of 7; delta kernel, dK/dV kernel writing dS,
  * dQ = dS K kernel): 2 bytes per (batch, q-head, query, key) plus 8 bytes per (batch, q-head, query),
  * in a buffer per device that belongs to the library, is allocated on first use, only grows and is
