@@ -630,8 +630,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
         p0 = keep_bit[E - 1] ? p0 * dst.scale : 0.f;              // :200-201
         p1 = keep_bit[E] ? p1 * dst.scale : 0.f;
       }
-      pb[E / 8][E % 8 - 1] = Tr::cvt(p0);     // p cast to dO's dtype (composed_tensors.py:191-193)
-      pb[E / 8][E % 8] = Tr::cvt(p1);
+      const typename Tr::p2_t p2 = Tr::cvt2(p0, p1);     // p cast to dO's dtype (composed_tensors.py:191-193)
+      pb[E / 8][E % 8 - 1] = p2[0];
+      pb[E / 8][E % 8] = p2[1];
     };
     auto ds_el = [&](int E) {
       const int mb = E / 16, i = E % 16, r = i % 4;
@@ -645,8 +646,9 @@ __device__ __forceinline__ void dkdv_item(const BwdArgs& a, const int hk, const 
       dp[mb][i] = s[mb][i] * (dpv - d4[(E / 4) & 1][r]);          // ds uses the undropped p (:242)
     };
     auto ds_pair = [&](int E) {  // E odd: ds cast to Q's dtype
-      sb[E / 8][E % 8 - 1] = Tr::cvt(dp[E / 16][E % 16 - 1]);
-      sb[E / 8][E % 8] = Tr::cvt(dp[E / 16][E % 16]);
+      const typename Tr::p2_t s2 = Tr::cvt2(dp[E / 16][E % 16 - 1], dp[E / 16][E % 16]);
+      sb[E / 8][E % 8 - 1] = s2[0];
+      sb[E / 8][E % 8] = s2[1];
     };
 
     // ---- dP = dO V^T, with p behind its MFMAs ------------------------------------
@@ -1259,8 +1261,9 @@ __device__ __forceinline__ void dq_item(const BwdArgs& a, const int h, const int
         if (n < si.seqlen_k) dbptr[(int64_t)n * a.sdb_n] = Tr::cvt(dsv);
       }
       if (E & 1) {   // ds cast to K's dtype, pair by pair
-        sb[E / 8][E % 8 - 1] = Tr::cvt(dp[mb][i - 1]);
-        sb[E / 8][E % 8] = Tr::cvt(dsv);
+        const typename Tr::p2_t s2 = Tr::cvt2(dp[mb][i - 1], dsv);
+        sb[E / 8][E % 8 - 1] = s2[0];
+        sb[E / 8][E % 8] = s2[1];
       }
     };
 

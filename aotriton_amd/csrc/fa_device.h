@@ -71,6 +71,10 @@ template <> struct Traits<bf16_t> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ bf16_t cvt(float x) { return (bf16_t)x; }
+  // two values at once: one v_cvt_pk_bf16_f32
+  static __device__ __forceinline__ p2_t cvt2(float x, float y) {
+    return __builtin_convertvector((vec<float, 2>){x, y}, p2_t);
+  }
 };
 
 template <> struct Traits<f16_t> {
@@ -84,6 +88,11 @@ template <> struct Traits<f16_t> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ f16_t cvt(float x) { return (f16_t)x; }
+  // two values at once: one v_cvt_pk_f16_f32 (from scalar conversions the compiler makes two
+  // v_cvt_f16_f32 and a v_pack_b32_f16)
+  static __device__ __forceinline__ p2_t cvt2(float x, float y) {
+    return __builtin_convertvector((vec<float, 2>){x, y}, p2_t);
+  }
 };
 
 // Eight accumulator values (i = 8*half .. 8*half+7) -> one MFMA operand.
@@ -91,7 +100,10 @@ template <typename T>
 __device__ __forceinline__ typename Traits<T>::op_t pack8(const f32x16& s, int half) {
   typename Traits<T>::op_t r;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) r[j] = Traits<T>::cvt(s[8 * half + j]);
+  for (int j = 0; j < 8; j += 2) {
+    const typename Traits<T>::p2_t p2 = Traits<T>::cvt2(s[8 * half + j], s[8 * half + j + 1]);
+    r[j] = p2[0]; r[j + 1] = p2[1];
+  }
   return r;
 }
 
