@@ -488,7 +488,7 @@ int validate_bwd(const fa_bwd_params* p, int32_t version, const fa_options* opt,
 hipError_t run_fwd(int dtype, int d, const fa::FwdArgs& a, const Shape& s, hipStream_t stream) {
   if (s.elementwise) return fa::run_fwd_valu(dtype, d, a, stream);
   if (dtype == FA_DTYPE_FLOAT32)
-    return d <= 256 ? fa::run_fwd_f32(d, a, s.windowed, s.bias, s.dropout, stream) : fa::run_fwd_valu(dtype, d, a, stream);
+    return fa::run_fwd_f32(d, a, s.windowed, s.bias, s.dropout, stream);
   if (d > 256) return fa::run_fwd_d512(dtype, a, s.windowed, s.bias, s.dropout, stream);
   const bool padded = a.head_dim != d || a.head_dim_v != d;   // head dim rounded up: the copies that mask the excess columns
   switch (d) {
@@ -601,11 +601,10 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   Shape s{};
   int e = validate_fwd(params, FA_FWD_PARAMS_VERSION, nullptr, &s);
   if (e != FA_SUCCESS) return e;
-  // the vector-ALU kernels (fp32) and the split-head-dim kernels (above 256): 32 rows per workgroup, 3-D grid
+  // the vector-ALU kernels (3-D grid), the fp32 kernels and the split-head-dim kernels (above 256)
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256 || s.elementwise;
   const fa::TileShape t = s.elementwise ? fa::TileShape{32, 1, 4, 0}
-                          : params->Q.dtype == FA_DTYPE_FLOAT32
-                              ? (s.d <= 256 ? fa::f32_tile_shape(s.d, -1) : fa::TileShape{32, 1, 4, 0})
+                          : params->Q.dtype == FA_DTYPE_FLOAT32 ? fa::f32_tile_shape(s.d, -1)
                           : s.d > 256 ? fa::d512_tile_shape(-1)
                                       : fa::fwd_tile_shape(params->Q.dtype, s.d, s.windowed);
   out->block_m = t.block_m; out->block_n = t.block_n; out->num_waves = t.num_waves;
@@ -613,7 +612,7 @@ int fa_query_fwd_config(const fa_fwd_params* params, int32_t num_cu, fa_kernel_c
   if (valu) {
     const int nz = s.num_seqlens != 0 ? std::abs(s.num_seqlens) : s.batch;
     const int mt = (s.max_sq + t.block_m - 1) / t.block_m;
-    if (s.elementwise || (params->Q.dtype == FA_DTYPE_FLOAT32 && s.d > 256)) {      // vector-ALU kernels: 3-D grid
+    if (s.elementwise) {      // vector-ALU kernels: 3-D grid
       out->grid[0] = mt; out->grid[1] = s.hq; out->grid[2] = nz;
     } else {      // one workgroup per tile, the tiles of a kv-head's group back to back on one XCD
       out->grid[0] = fa::kNumXcd * ((nz * s.hk + fa::kNumXcd - 1) / fa::kNumXcd) * (s.hq / s.hk) * mt;
@@ -655,7 +654,7 @@ int fa_query_bwd_config(const fa_bwd_params* params, const fa_options* options, 
   const bool valu = params->Q.dtype == FA_DTYPE_FLOAT32 || s.d > 256 || s.elementwise;   // vector-ALU kernels: 32 rows per workgroup
   if (valu && kernel_slot == 3) return FA_ERROR_PEER_ACCESS_UNSUPPORTED;
   const bool split_d = !s.elementwise && params->Q.dtype != FA_DTYPE_FLOAT32 && s.d > 256 && kernel_slot != 0;
-  const bool f32_mfma = !s.elementwise && params->Q.dtype == FA_DTYPE_FLOAT32 && s.d <= 256 && kernel_slot != 0;
+  const bool f32_mfma = !s.elementwise && params->Q.dtype == FA_DTYPE_FLOAT32 && kernel_slot != 0;
   const fa::TileShape t = f32_mfma ? fa::f32_tile_shape(s.d, kernel_slot)
                           : split_d ? fa::d512_tile_shape(kernel_slot)
                           : valu  ? (kernel_slot == 1 ? fa::TileShape{1, 32, 4, 0} : fa::TileShape{32, 1, 4, 0})
@@ -977,7 +976,7 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
     }
     a.delta = static_cast<float*>(delta.ptr);
     const bool slow = s.elementwise;              // rows moved element by element: vector-ALU kernels
-    const bool f32 = !slow && dt == FA_DTYPE_FLOAT32;      // fp32 MFMA kernels up to head dim 256, vector-ALU kernels above
+    const bool f32 = !slow && dt == FA_DTYPE_FLOAT32;      // fp32 MFMA kernels
     const bool big = !slow && !f32 && s.d > 256;  // head dim split over the waves
     // fp32 and the head dims above 256 take delta from the vector-ALU kernel.  The dQ kernel of the
     // 16-bit types up to head dim 256 computes delta from the O and dO rows it holds and writes it
@@ -1047,8 +1046,7 @@ static int attn_bwd_impl(const fa_bwd_params* p_in, int32_t params_version, void
       if (slow)
         err = fa::run_bwd_valu(dt, s.d, slot, a, stream);
       else if (f32)
-        err = s.d <= 256 ? fa::run_bwd_f32(s.d, slot, a, s.windowed, s.bias, s.dropout, stream)
-                         : fa::run_bwd_valu(dt, s.d, slot, a, stream);
+        err = fa::run_bwd_f32(s.d, slot, a, s.windowed, s.bias, s.dropout, stream);
       else if (big)
         err = fa::run_bwd_d512(dt, slot, a, s.windowed, s.bias, s.dropout, stream);
       else

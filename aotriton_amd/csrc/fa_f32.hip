@@ -1,4 +1,4 @@
-// MFMA kernels for fp32 tensors (v_mfma_f32_32x32x2_f32), head dims up to 256, gfx950.
+// MFMA kernels for fp32 tensors (v_mfma_f32_32x32x2_f32), head dims up to 512, gfx950.
 //
 // The reference compiles its kernels for fp32 tensors as well ('*fp32:16' among the tensor types of
 // modules/flash/aot/_common.py:10-14); these compute what the 16-bit kernels of this library do
@@ -19,8 +19,11 @@
 // The structure is that of the kernels for head dims above 256 (fa_d512.hip): the head dim is
 // split over four waves that work on the same 32 rows, the GEMMs that contract over the head dim
 // exchange 32 x 32 partial blocks through LDS, and in the backward each wave does a quarter of the
-// element work and hands P and dS on.  Compiled for 128 and 256 columns (smaller head dims
-// zero-filled); fp32 at head dims above 256 stays on the vector-ALU kernels.
+// element work and hands P and dS on.  Compiled for 128, 256 and 512 columns (smaller head dims
+// zero-filled).  At 512 columns two staged tiles fill 128 KB of the 160 KB of LDS: the forward and
+// the dQ kernel then run one 32-row block per workgroup instead of two, and the partial blocks of
+// S and dP go through ONE area one after the other (two more barriers per tile, next to 256 MFMAs
+// of 64 cycles per wave).
 #include "fa_device.h"
 #include "fa_kernels.h"
 
@@ -30,9 +33,6 @@ namespace {
 constexpr int kNW = 4;           // waves per 32-row block
 constexpr int kBC = 32;          // rows of the streamed tiles per step
 constexpr int kNT = kNW * 64;
-constexpr int kRB = 2;           // 32-row blocks per workgroup (forward, dQ)
-constexpr int kBR2 = 32 * kRB;
-constexpr int kNT2 = kRB * kNT;
 constexpr int kPartBytes = kNW * 64 * 16 * 4;     // one partial block per wave
 constexpr int kOpndBytes = 4 * 64 * 16;           // one block of P or dS: 4 quarters x 64 lanes x 4 floats
 
@@ -43,6 +43,11 @@ struct Cfg {
   static constexpr int DB = DW / 32;      // 32-column blocks a wave owns
   static constexpr int STR = D;           // floats per tile row in LDS (unpadded, pieces swizzled)
   static constexpr int TILE_BYTES = kBC * STR * 4;
+  static constexpr int RB = D > 256 ? 1 : 2;      // 32-row blocks per workgroup (forward, dQ)
+  static constexpr int BR = 32 * RB;
+  static constexpr int NT = RB * kNT;
+  static constexpr bool ONE_PART = D > 256;       // S and dP partial blocks share one area
+  static constexpr int PARTS = ONE_PART ? 1 : 2;
 };
 
 // LDS tiles keep the 16-byte piece q of row r at piece position q ^ swz(r).  Two access patterns must
@@ -140,6 +145,9 @@ __device__ __forceinline__ f32x16 row_gemm(const float* tile, int c, int hi, int
     const f32x4 a4 = *reinterpret_cast<const f32x4*>(p + ((q0 + 2 * j) ^ sw) * 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc = mfma32(a4[e], res[j][e], acc);
+    // at 512 columns the registers are full of accumulators and resident operands: keep the
+    // scheduler from requesting all sixteen pieces of the row up front
+    if (Cfg<D>::KJ > 8 && j % 4 == 3) __builtin_amdgcn_sched_barrier(0);
   }
   return acc;
 }
@@ -154,6 +162,7 @@ __device__ __forceinline__ void col_gemm(const float* tile, int c, int hi, int c
     const int q0 = (col0 + c) / 4, sw = swz(r);
 #pragma unroll
     for (int db = 0; db < Cfg<D>::DB; ++db) acc[db] = mfma32(p[((q0 + 8 * db) ^ sw) * 4], x[i], acc[db]);
+    if (Cfg<D>::KJ > 8 && i % 4 == 3) __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -168,17 +177,17 @@ __device__ __forceinline__ Window window_of(const MaskArgs& m, int sq, int sk) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// forward: one workgroup = 64 query rows of one head = 8 waves, four per 32-row block
+// forward: one workgroup = 64 (at 512 columns: 32) query rows of one head, four waves per 32-row block
 // ---------------------------------------------------------------------------------------------
 template <int D>
 struct SmemFwd {
   static constexpr int V_OFF = Cfg<D>::TILE_BYTES;
   static constexpr int PART_OFF = 2 * Cfg<D>::TILE_BYTES;
-  static constexpr int BYTES = PART_OFF + kRB * kPartBytes;
+  static constexpr int BYTES = PART_OFF + Cfg<D>::RB * kPartBytes;
 };
 
 template <int D, bool kWindowed, bool kBias, bool kDropout>
-__global__ __launch_bounds__(kNT2) void fwd_f32_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(Cfg<D>::NT) void fwd_f32_kernel(const FwdArgs a) {
   using C = Cfg<D>;
   using SM = SmemFwd<D>;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -191,7 +200,7 @@ __global__ __launch_bounds__(kNT2) void fwd_f32_kernel(const FwdArgs a) {
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
   // one workgroup per (sequence, q-head, Q tile): the tiles of a kv-head's group back to back on one
   // XCD, most visible keys (causal) first
-  const int nmt = (a.seq.max_seqlen_q + kBR2 - 1) / kBR2, group = a.hq / a.hk;
+  const int nmt = (a.seq.max_seqlen_q + C::BR - 1) / C::BR, group = a.hq / a.hk;
   int pair, r_item;
   if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, group * nmt, pair, r_item)) return;
   const int z = pair / a.hk, h = (pair % a.hk) * group + r_item % group;
@@ -207,10 +216,10 @@ __global__ __launch_bounds__(kNT2) void fwd_f32_kernel(const FwdArgs a) {
   }
 
   const SeqInfo si = get_seq(a.seq, z);
-  const int q0 = mt * kBR2;
+  const int q0 = mt * C::BR;
   if (q0 >= si.seqlen_q) return;
   const Window w = window_of<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
-  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kBR2, kBC);
+  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, C::BR, kBC);
 
   const int hk = h / (a.hq / a.hk);                       // fwd_kernel.py:360
   const int row = q0 + 32 * rb + c;                       // this lane's query row (the same in the four waves of a row block)
@@ -245,7 +254,7 @@ __global__ __launch_bounds__(kNT2) void fwd_f32_kernel(const FwdArgs a) {
   const float* vt = reinterpret_cast<const float*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                     (int64_t)(si.k_start + br.lo * kBC) * a.sv.s;
   int rows_left = si.seqlen_k - br.lo * kBC;      // > 0
-  TileFetch<D, kNT2> kf, vf;
+  TileFetch<D, C::NT> kf, vf;
   auto fetch = [&]() {
     const int rows = rows_left < kBC ? rows_left : kBC;
     kf.load(kt, rows, a.sk.s, d_qk, tid);
@@ -385,7 +394,7 @@ template <int D>
 struct SmemDkDv {
   static constexpr int STAT_OFF = 2 * Cfg<D>::TILE_BYTES;
   static constexpr int PART_OFF = STAT_OFF + 2 * kBC * 4;
-  static constexpr int OPND_OFF = PART_OFF + 2 * kPartBytes;
+  static constexpr int OPND_OFF = PART_OFF + Cfg<D>::PARTS * kPartBytes;
   static constexpr int BYTES = OPND_OFF + 2 * kOpndBytes;
 };
 
@@ -399,7 +408,7 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_f32_kernel(const BwdArgs a) {
   float* Ls = reinterpret_cast<float*>(smem_raw + SM::STAT_OFF);
   float* Ds = Ls + kBC;
   float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF);
-  float* partD = partS + kPartBytes / 4;
+  float* partD = C::ONE_PART ? partS : partS + kPartBytes / 4;
   float* opP = reinterpret_cast<float*>(smem_raw + SM::OPND_OFF);
   float* opS = opP + kOpndBytes / 4;
 
@@ -497,12 +506,22 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_f32_kernel(const BwdArgs a) {
       for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
       s = row_gemm<D>(Qs, c, hi, col0, kreg, s);
       dp = row_gemm<D>(dOs, c, hi, col0, vreg, dp);
-      part_write(partS, wave, lane, s);
-      part_write(partD, wave, lane, dp);
-      __syncthreads();
       // this wave's quarter of the elements: queries m0 + 8 wave + 4 hi + r
-      const f32x4 s4 = part_sum_quarter(partS, wave, lane);
-      const f32x4 dp4 = part_sum_quarter(partD, wave, lane);
+      f32x4 s4, dp4;
+      part_write(partS, wave, lane, s);
+      if constexpr (C::ONE_PART) {
+        __syncthreads();
+        s4 = part_sum_quarter(partS, wave, lane);
+        __syncthreads();               // S has been read: dP goes through the same area
+        part_write(partD, wave, lane, dp);
+        __syncthreads();
+        dp4 = part_sum_quarter(partD, wave, lane);
+      } else {
+        part_write(partD, wave, lane, dp);
+        __syncthreads();
+        s4 = part_sum_quarter(partS, wave, lane);
+        dp4 = part_sum_quarter(partD, wave, lane);
+      }
 
       DropoutState dst{};
       if (kDropout) dst = dropout_for_head(drop0, z, hq, a.hq, a.seq.max_seqlen_q);
@@ -570,18 +589,18 @@ __global__ __launch_bounds__(kNT) void bwd_dkdv_f32_kernel(const BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// dQ and dB: one workgroup = 64 query rows of one head = 8 waves, four per 32-row block; the lane's
+// dQ and dB: one workgroup = 64 (at 512 columns: 32) query rows of one head, four waves per 32-row block; the lane's
 // query is lane % 32 of its row block, the keys of a tile are spread over the accumulator elements
 // ---------------------------------------------------------------------------------------------
 template <int D>
 struct SmemDq {
   static constexpr int PART_OFF = 2 * Cfg<D>::TILE_BYTES;
-  static constexpr int OPND_OFF = PART_OFF + kRB * 2 * kPartBytes;
-  static constexpr int BYTES = OPND_OFF + kRB * kOpndBytes;
+  static constexpr int OPND_OFF = PART_OFF + Cfg<D>::RB * Cfg<D>::PARTS * kPartBytes;
+  static constexpr int BYTES = OPND_OFF + Cfg<D>::RB * kOpndBytes;
 };
 
 template <int D, bool kWindowed, bool kBias, bool kDropout>
-__global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(Cfg<D>::NT) void bwd_dq_f32_kernel(const BwdArgs a) {
   using C = Cfg<D>;
   using SM = SmemDq<D>;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
@@ -594,22 +613,22 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
   const int lane = tid & 63, c = lane & 31, hi = lane >> 5;
   // one workgroup per (sequence, q-head, Q tile): the tiles of a kv-head's group back to back on one
   // XCD, most visible keys (causal) first
-  const int nmt = (a.seq.max_seqlen_q + kBR2 - 1) / kBR2, group = a.hq / a.hk;
+  const int nmt = (a.seq.max_seqlen_q + C::BR - 1) / C::BR, group = a.hq / a.hk;
   int pair, r_item;
   if (!xcd_item(blockIdx.x, nseq_of(a.seq, a.batch) * a.hk, group * nmt, pair, r_item)) return;
   const int z = pair / a.hk, h = (pair % a.hk) * group + r_item % group;
   const int mt = nmt - 1 - r_item / group;
   const int d_qk = a.head_dim, d_v = a.head_dim_v;
   const int col0 = cw * C::DW;
-  float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * 2 * (kPartBytes / 4);
-  float* partD = partS + kPartBytes / 4;
+  float* partS = reinterpret_cast<float*>(smem_raw + SM::PART_OFF) + rb * C::PARTS * (kPartBytes / 4);
+  float* partD = C::ONE_PART ? partS : partS + kPartBytes / 4;
   float* opS = reinterpret_cast<float*>(smem_raw + SM::OPND_OFF) + rb * (kOpndBytes / 4);
 
   const SeqInfo si = get_seq(a.seq, z);
-  const int q0 = mt * kBR2;
+  const int q0 = mt * C::BR;
   if (q0 >= si.seqlen_q) return;
   const Window w = window_of<kWindowed>(a.mask, si.seqlen_q, si.seqlen_k);
-  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, kBR2, kBC);
+  const BlockRanges br = block_ranges(kWindowed, w.left, w.right, q0, si.seqlen_q, si.seqlen_k, C::BR, kBC);
 
   const int hk = h / (a.hq / a.hk);
   const int row = q0 + 32 * rb + c;
@@ -627,7 +646,7 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
     if (!want_db) return;
     const int c0 = j_from * kBC, c1 = j_to * kBC < si.seqlen_k ? j_to * kBC : si.seqlen_k;
     if (c0 >= c1) return;
-    for (int rr = wave; rr < kBR2; rr += kRB * kNW) {
+    for (int rr = wave; rr < C::BR; rr += C::RB * kNW) {
       const int m = q0 + rr;
       if (m >= si.seqlen_q) break;
       float* rowp = dbhead + (int64_t)m * a.sdb_m;
@@ -675,7 +694,7 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
     const float* vt = reinterpret_cast<const float*>(a.v) + (int64_t)si.batch_index * a.sv.z + (int64_t)hk * a.sv.h +
                       (int64_t)(si.k_start + br.lo * kBC) * a.sv.s;
     int rows_left = si.seqlen_k - br.lo * kBC;      // > 0
-    TileFetch<D, kNT2> kf, vf;
+    TileFetch<D, C::NT> kf, vf;
     auto fetch = [&]() {
       const int rows = rows_left < kBC ? rows_left : kBC;
       kf.load(kt, rows, a.sk.s, d_qk, tid);
@@ -695,12 +714,22 @@ __global__ __launch_bounds__(kNT2) void bwd_dq_f32_kernel(const BwdArgs a) {
       for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
       s = row_gemm<D>(Ks, c, hi, col0, qreg, s);
       dp = row_gemm<D>(Vs, c, hi, col0, doreg, dp);
-      part_write(partS, cw, lane, s);
-      part_write(partD, cw, lane, dp);
-      __syncthreads();
       // this wave's quarter of its row block's elements: keys j kBC + 8 cw + 4 hi + r
-      const f32x4 s4 = part_sum_quarter(partS, cw, lane);
-      const f32x4 dp4 = part_sum_quarter(partD, cw, lane);
+      f32x4 s4, dp4;
+      part_write(partS, cw, lane, s);
+      if constexpr (C::ONE_PART) {
+        __syncthreads();
+        s4 = part_sum_quarter(partS, cw, lane);
+        __syncthreads();               // S has been read: dP goes through the same area
+        part_write(partD, cw, lane, dp);
+        __syncthreads();
+        dp4 = part_sum_quarter(partD, cw, lane);
+      } else {
+        part_write(partD, cw, lane, dp);
+        __syncthreads();
+        s4 = part_sum_quarter(partS, cw, lane);
+        dp4 = part_sum_quarter(partD, cw, lane);
+      }
 
       const bool masked = !br.is_full(j);
       const unsigned m_d = m_none ? 0x40000000u : (unsigned)(j * kBC + 8 * cw + 4 * hi - m_lo);
@@ -779,8 +808,8 @@ hipError_t launch(dim3 grid, int smem, hipStream_t stream, const Args& a) {
 
 template <int D>
 hipError_t run_fwd_d(const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
-  const dim3 grid(xcd_grid(nseq_of(a.seq, a.batch) * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + kBR2 - 1) / kBR2)));
-#define FA_CALL(W, B, P) launch<fwd_f32_kernel<D, W, B, P>, kNT2>(grid, SmemFwd<D>::BYTES, s, a)
+  const dim3 grid(xcd_grid(nseq_of(a.seq, a.batch) * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + Cfg<D>::BR - 1) / Cfg<D>::BR)));
+#define FA_CALL(W, B, P) launch<fwd_f32_kernel<D, W, B, P>, Cfg<D>::NT>(grid, SmemFwd<D>::BYTES, s, a)
   FA_F32_SWITCH(FA_CALL)
 #undef FA_CALL
 }
@@ -795,8 +824,8 @@ hipError_t run_bwd_d(int kernel_slot, const BwdArgs& a, bool windowed, bool bias
 #undef FA_CALL
   }
   if (kernel_slot == 2) {
-    const dim3 grid(xcd_grid(nseq * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + kBR2 - 1) / kBR2)));
-#define FA_CALL(W, B, P) launch<bwd_dq_f32_kernel<D, W, B, P>, kNT2>(grid, SmemDq<D>::BYTES, s, a)
+    const dim3 grid(xcd_grid(nseq * a.hk, (a.hq / a.hk) * ((a.seq.max_seqlen_q + Cfg<D>::BR - 1) / Cfg<D>::BR)));
+#define FA_CALL(W, B, P) launch<bwd_dq_f32_kernel<D, W, B, P>, Cfg<D>::NT>(grid, SmemDq<D>::BYTES, s, a)
     FA_F32_SWITCH(FA_CALL)
 #undef FA_CALL
   }
@@ -809,6 +838,7 @@ hipError_t run_bwd_d(int kernel_slot, const BwdArgs& a, bool windowed, bool bias
 hipError_t run_fwd_f32(int head_dim, const FwdArgs& a, bool windowed, bool bias, bool dropout, hipStream_t s) {
   if (head_dim <= 128) return run_fwd_d<128>(a, windowed, bias, dropout, s);
   if (head_dim == 256) return run_fwd_d<256>(a, windowed, bias, dropout, s);
+  if (head_dim == 512) return run_fwd_d<512>(a, windowed, bias, dropout, s);
   return hipErrorNotSupported;
 }
 
@@ -816,16 +846,22 @@ hipError_t run_bwd_f32(int head_dim, int kernel_slot, const BwdArgs& a, bool win
                        hipStream_t s) {
   if (head_dim <= 128) return run_bwd_d<128>(kernel_slot, a, windowed, bias, dropout, s);
   if (head_dim == 256) return run_bwd_d<256>(kernel_slot, a, windowed, bias, dropout, s);
+  if (head_dim == 512) return run_bwd_d<512>(kernel_slot, a, windowed, bias, dropout, s);
   return hipErrorNotSupported;
 }
 
-TileShape f32_tile_shape(int head_dim, int kernel_slot) {
-  // forward (kernel_slot < 0) and dQ: 64 queries per workgroup against 32 keys per step; dK/dV: 32
+template <int D>
+static TileShape tile_shape_d(int kernel_slot) {
+  // forward (kernel_slot < 0) and dQ: the workgroup's queries against 32 keys per step; dK/dV: 32
   // keys per workgroup against 32 queries per step
-  const bool wide = head_dim > 128;
-  if (kernel_slot < 0) return TileShape{kBR2, kBC, kRB * kNW, wide ? SmemFwd<256>::BYTES : SmemFwd<128>::BYTES};
-  if (kernel_slot == 2) return TileShape{kBR2, kBC, kRB * kNW, wide ? SmemDq<256>::BYTES : SmemDq<128>::BYTES};
-  return TileShape{kBC, kBC, kNW, wide ? SmemDkDv<256>::BYTES : SmemDkDv<128>::BYTES};
+  if (kernel_slot < 0) return TileShape{Cfg<D>::BR, kBC, Cfg<D>::RB * kNW, SmemFwd<D>::BYTES};
+  if (kernel_slot == 2) return TileShape{Cfg<D>::BR, kBC, Cfg<D>::RB * kNW, SmemDq<D>::BYTES};
+  return TileShape{kBC, kBC, kNW, SmemDkDv<D>::BYTES};
+}
+
+TileShape f32_tile_shape(int head_dim, int kernel_slot) {
+  return head_dim <= 128 ? tile_shape_d<128>(kernel_slot)
+         : head_dim <= 256 ? tile_shape_d<256>(kernel_slot) : tile_shape_d<512>(kernel_slot);
 }
 
 }  // namespace fa

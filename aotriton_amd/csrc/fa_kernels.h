@@ -50,7 +50,8 @@ hipError_t run_bwd_f32(int head_dim, int kernel_slot, const BwdArgs& a, bool win
                        hipStream_t s);
 TileShape f32_tile_shape(int head_dim, int kernel_slot);
 
-// Vector-ALU kernels (no MFMA): fp32 tensors at any head dim, every type at head dim 512.
+// Vector-ALU kernels (no MFMA): every type at every compiled head dim; they serve tensors whose
+// rows the MFMA kernels cannot load in 16-byte pieces, and delta of the fp32 and split-head-dim families.
 // head_dim is the compiled one (64, 128, 256, 512).  kernel_slot of the backward: 0 delta,
 // 1 dK/dV, 2 dQ and dB.
 hipError_t run_fwd_valu(int dtype, int head_dim, const FwdArgs& a, hipStream_t s);

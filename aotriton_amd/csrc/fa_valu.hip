@@ -1,6 +1,7 @@
 // Plain vector-ALU kernels, one row of Q (or of K) per group of 8 lanes: the functional path
-// for what the MFMA kernels do not cover, i.e. fp32 tensors (any head dim) and head dims
-// above 256 up to 512 (any type).
+// for what the MFMA kernels do not cover, i.e. tensors whose rows are not made of aligned 16-byte
+// pieces (loads and stores element by element), and delta for the fp32 kernels and the kernels
+// of head dims above 256.
 //
 // The reference compiles its Triton kernels for fp32 and for head dim 512 as well
 // (modules/flash/aot/_common.py:10-14 lists the head dims, '*fp32:16' is among the tensor

@@ -146,7 +146,7 @@ def test_fp32_baseline_config_1():
     dict(D=40, causal=False, Dv=72, Hk=1, sq=77, sk=129), dict(D=128, causal=1, sq=300, sk=140),
 ])
 def test_fp32_inputs(case):
-    # fp32 tensors run on the fp32 MFMA kernels (vector-ALU kernels above head dim 256); the oracle is fp64 against fp32
+    # fp32 tensors run on the fp32 MFMA kernels; the oracle is fp64 against fp32
     c = dict(Hk=4, sq=128, sk=128, bias=False, dropout_p=0.0, bshd=False, Dv=None)
     c.update(case)
     _run_case(2, 4, c['Hk'], c['sq'], c['sk'], c['D'], torch.float32, c['causal'], dropout_p=c['dropout_p'],
@@ -155,10 +155,11 @@ def test_fp32_inputs(case):
 
 @pytest.mark.parametrize('causal', [False, True, (70, 33)])
 @pytest.mark.parametrize('D,Dv,p,bias', [(128, None, 0.0, False), (256, 200, 0.1, False), (72, 256, 0.0, True),
-                                         (192, None, 0.3, True)])
+                                         (192, None, 0.3, True), (512, None, 0.0, False), (384, 272, 0.1, False),
+                                         (264, 512, 0.0, True), (448, None, 0.3, True)])
 def test_fp32_mfma_kernels(causal, D, Dv, p, bias):
     # several 32-row tiles each way, ragged ends, grouped heads, every combination of mask, bias
-    # (with dB) and dropout, on both compiled widths (128 and 256 columns)
+    # (with dB) and dropout, on the three compiled widths (128, 256 and 512 columns)
     if bias and causal is True:
         causal = (1000, 0)       # the same mask through the window arguments
     _run_case(2, 6, 2, 203, 261, D, torch.float32, causal, Dv=Dv, dropout_p=p, bias=bias, bwd_backend=0)
@@ -168,7 +169,7 @@ def test_fp32_mfma_kernels(causal, D, Dv, p, bias):
 @pytest.mark.parametrize('D,Dv', [(512, None), (320, 264), (128, 512)])
 def test_head_dims_up_to_512(dtype, D, Dv):
     # above 256 the 16-bit types run on the kernels that split the head dim over the waves, fp32 on
-    # the vector-ALU kernels (fp32 up to 256: fp32 MFMA kernels) (the reference compiles head dim 512, modules/flash/aot/_common.py:10-14)
+    # the 512-column build of its MFMA kernels (the reference compiles head dim 512, modules/flash/aot/_common.py:10-14)
     _run_case(1, 4, 2, 150, 131, D, dtype, (40, 0), Dv=Dv, bwd_backend=0)
 
 
@@ -282,7 +283,7 @@ def _sampled_grid_cases(n=72, seed=2024):
         if p > 0.0 and sq * sk > 600 * 600:
             p = 0.0
         if dtype == torch.float32 and max(D, Dv or 0) > 256 and sq * sk > 1024 * 1024:
-            sq, sk = min(sq, 512), min(sk, 512)      # vector-ALU kernels: keep the case short
+            sq, sk = min(sq, 512), min(sk, 512)      # keep the fp64 oracle of the case short
         split_only = dtype == torch.float32 or max(D, Dv or 0) > 256
         backend = 0 if split_only else rnd.choice([0, 1])
         cases.append((fam, heads, D, Dv, sq, sk, causal, p, dtype, flip, bias, scale, backend))
