@@ -28,6 +28,9 @@ COMMON = [
 # Per-file additions.  The dQ kernels post-process MFMA results with the vector ALU; letting
 # the register allocator keep those results in VGPRs saves the AGPR read per element.
 EXTRA = {
+    # the ILP-first scheduling strategy: dK/dV kernel of the headline shape -1..2 % (same-box A/B,
+    # no spills either way); level on the forward and the dQ-from-dS kernel, which keep the default
+    'fa_bwd_dkdv_d128.hip': ['-mllvm', '-amdgpu-sched-strategy=max-ilp'],
     'fa_bwd_dq_d64.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
     'fa_bwd_dq_d128.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form'],
 }
