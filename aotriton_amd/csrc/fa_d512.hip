@@ -130,13 +130,17 @@ struct TileFetch {
 // A K/V tile of 32 keys is 64 KB; with 32 rows per workgroup that is 32 FLOP per byte streamed and
 // the kernel runs at the rate the L2 delivers K/V (about 225 TFLOP/s).  Two row blocks share the
 // tile here; each has its own four waves (one per 128 columns), so a SIMD holds two waves and one
-// covers the other's waits.  One K/V stage in LDS, the next tile waits in registers.
+// covers the other's waits.  Two K stages and one V stage in LDS, the next tile waits in registers:
+// K of the next tile is published behind the PV MFMAs (its stage was last read a tile ago), V behind
+// the barrier that ends the tile, where it becomes visible with the next tile's partial blocks; two
+// barriers per tile.
 constexpr int kFRB = 2;              // 32-row blocks per workgroup
 constexpr int kFBR = 32 * kFRB;      // query rows per workgroup
 constexpr int kFNT = kFRB * kNT;     // threads per workgroup
 struct SmemFwd512 {
   static constexpr int ASTR = Smem512::ASTR, BSTR = Smem512::BSTR;
-  static constexpr int V_OFF = Smem512::A_ELEMS * 2;
+  static constexpr int K_STAGE = Smem512::A_ELEMS * 2;       // bytes of one K stage; there are two
+  static constexpr int V_OFF = 2 * K_STAGE;
   static constexpr int PART_OFF = V_OFF + Smem512::B_ELEMS * 2;
   static constexpr int BYTES = PART_OFF + kFRB * Smem512::PART_BYTES;
 };
@@ -230,10 +234,8 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
     vf.load(vt, rows, a.sv.s, d_v, tid);
     kt += (int64_t)kBC * a.sk.s; vt += (int64_t)kBC * a.sv.s; rows_left -= kBC;
   };
-  auto publish = [&]() {
-    kf.store(Ks, SM::ASTR, tid);
-    vf.store(Vs, SM::BSTR, tid);
-  };
+  auto publish_k = [&](int stage) { kf.store(Ks + stage * Smem512::A_ELEMS, SM::ASTR, tid); };
+  auto publish_v = [&]() { vf.store(Vs, SM::BSTR, tid); };
 
   const T* bptr = nullptr;
   if (kBias)
@@ -267,15 +269,17 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
   const int v_lane = (4 * hi + (lane & 15) / 4) * SM::BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + col0;
 
   fetch();
-  publish();
+  publish_k(0);
+  publish_v();
   __syncthreads();
   for (int j = br.lo; j <= br.hi; ++j) {
+    const int stage = (j - br.lo) & 1;
     if (j < br.hi) fetch();
     // this wave's share of S^T = K Q^T
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    const T* ks = Ks + c * SM::ASTR + col0 + hi * 8;
+    const T* ks = Ks + stage * Smem512::A_ELEMS + c * SM::ASTR + col0 + hi * 8;
 #pragma unroll
     for (int k = 0; k < kKS; ++k) s = Tr::mfma(*reinterpret_cast<const op_t*>(ks + k * 16), qreg[k], s);
     part_write(part, cw, lane, s);
@@ -343,11 +347,9 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
       for (int db = 0; db < kDB; ++db)
         o[db] = Tr::mfma(lds_read_tr8<T>(vs + t * 16 * SM::BSTR + db * 32, SM::BSTR), pb, o[db]);
     }
-    __syncthreads();                 // the tile and the partial blocks have been read
-    if (j < br.hi) {
-      publish();
-      __syncthreads();
-    }
+    if (j < br.hi) publish_k(stage ^ 1);
+    __syncthreads();                 // V and the partial blocks have been read, the next K is in place
+    if (j < br.hi) publish_v();      // (visible behind the barrier that follows the next partial blocks)
   }
 
   const float l = cross_sum(l_i);
