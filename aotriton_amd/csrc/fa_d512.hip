@@ -274,7 +274,6 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
   __syncthreads();
   for (int j = br.lo; j <= br.hi; ++j) {
     const int stage = (j - br.lo) & 1;
-    if (j < br.hi) fetch();
     // this wave's share of S^T = K Q^T
     f32x16 s;
 #pragma unroll
@@ -282,6 +281,10 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
     const T* ks = Ks + stage * Smem512::A_ELEMS + c * SM::ASTR + col0 + hi * 8;
 #pragma unroll
     for (int k = 0; k < kKS; ++k) s = Tr::mfma(*reinterpret_cast<const op_t*>(ks + k * 16), qreg[k], s);
+    // behind the MFMAs: V of this tile goes to its stage (read behind the next barrier), then the
+    // staging registers take the next tile
+    if (j > br.lo) publish_v();
+    if (j < br.hi) fetch();
     part_write(part, cw, lane, s);
     __syncthreads();
     s = part_sum(part, lane);
@@ -349,7 +352,6 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
     }
     if (j < br.hi) publish_k(stage ^ 1);
     __syncthreads();                 // V and the partial blocks have been read, the next K is in place
-    if (j < br.hi) publish_v();      // (visible behind the barrier that follows the next partial blocks)
   }
 
   const float l = cross_sum(l_i);
