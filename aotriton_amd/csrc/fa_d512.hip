@@ -69,6 +69,40 @@ __device__ __forceinline__ f32x16 part_sum(const float* area, int lane) {
   return x;
 }
 
+// The same sum with the wave's own block taken from its registers instead of from LDS (the values
+// are the ones it wrote, the order of the additions is unchanged, so the result is the same bit for
+// bit in all four waves): a quarter less to read.
+template <int W>
+__device__ __forceinline__ f32x16 part_sum_own_w(const float* area, int lane, const f32x16& own) {
+  f32x16 x;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    f32x4 acc;
+#pragma unroll
+    for (int w = 0; w < kNW; ++w) {
+      f32x4 t;
+      if (w == W) t = f32x4{own[4 * g], own[4 * g + 1], own[4 * g + 2], own[4 * g + 3]};
+      else t = *reinterpret_cast<const f32x4*>(area + ((w * 4 + g) * 64 + lane) * 4);
+      if (w == 0) acc = t;
+      else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += t[r];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) x[4 * g + r] = acc[r];
+  }
+  return x;
+}
+__device__ __forceinline__ f32x16 part_sum_own(const float* area, int wave, int lane, const f32x16& own) {
+  switch (wave) {      // (the wave index is a scalar)
+    case 0: return part_sum_own_w<0>(area, lane, own);
+    case 1: return part_sum_own_w<1>(area, lane, own);
+    case 2: return part_sum_own_w<2>(area, lane, own);
+    default: return part_sum_own_w<3>(area, lane, own);
+  }
+}
+
 // Backward: the element work on a summed block needs no row reduction, so it is split as well:
 // wave g adds only elements 4 g .. 4 g + 3 of every lane (a quarter of each partial block), does the
 // exponentials, mask, dropout and dS for those, and hands the two results to all waves as 16-bit
@@ -287,7 +321,7 @@ __global__ __launch_bounds__(kFNT) void fwd_d512_kernel(const FwdArgs a) {
     if (j < br.hi) fetch();
     part_write(part, cw, lane, s);
     __syncthreads();
-    s = part_sum(part, lane);
+    s = part_sum_own(part, cw, lane, s);
 
     // scale, bias and mask on the raw scores
     if (prescale) {
