@@ -185,6 +185,15 @@ def test_split_head_dim_kernels(dtype, causal, D, Dv, p, bias):
     _run_case(2, 6, 2, 203, 261, D, dtype, causal, Dv=Dv, dropout_p=p, bias=bias, bwd_backend=0)
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('sk', [1, 31, 33, 64, 65])
+def test_head_dim_512_with_one_to_three_key_tiles(dtype, sk):
+    # the kernels of head dims above 256 stream 32-key tiles through two K stages: one tile (nothing to
+    # prefetch), two (each stage used once) and three (the first stage reused)
+    _run_case(1, 2, 1, 70, sk, 512, dtype, False, bwd_backend=0)
+    _run_case(1, 2, 1, 70, sk, 384, dtype, (1000, 5), bwd_backend=0)
+
+
 def test_head_dim_512_with_bias_and_dropout():
     _run_case(1, 2, 2, 100, 100, 512, torch.bfloat16, True, dropout_p=0.2, bias=True, bwd_backend=0)
 
