@@ -179,10 +179,17 @@ __device__ __forceinline__ Window window_of(const MaskArgs& m, int sq, int sk) {
 // ---------------------------------------------------------------------------------------------
 // forward: one workgroup = 64 (at 512 columns: 32) query rows of one head, four waves per 32-row block
 // ---------------------------------------------------------------------------------------------
+// At 128 columns there are two K stages: K of the next tile is published behind the PV MFMAs of
+// the current one (that stage was last read a tile earlier), V of a tile behind the QK MFMAs of the
+// same tile (the V stage was released by the barrier that ended the tile before, and is read behind
+// the partial-block barrier), so a tile costs two barriers (forward + 2.5-4.5 %: 110 -> 115 TFLOP/s
+// at B4 H32 S4096).  At 256 columns the same schedule measures 1 % slower and at 512 a second K
+// stage does not fit; there the next tile is published between two barriers of its own.
 template <int D>
 struct SmemFwd {
-  static constexpr int V_OFF = Cfg<D>::TILE_BYTES;
-  static constexpr int PART_OFF = 2 * Cfg<D>::TILE_BYTES;
+  static constexpr int K_STAGES = D > 128 ? 1 : 2;
+  static constexpr int V_OFF = K_STAGES * Cfg<D>::TILE_BYTES;
+  static constexpr int PART_OFF = V_OFF + Cfg<D>::TILE_BYTES;
   static constexpr int BYTES = PART_OFF + Cfg<D>::RB * kPartBytes;
 };
 
@@ -261,7 +268,9 @@ __global__ __launch_bounds__(Cfg<D>::NT) void fwd_f32_kernel(const FwdArgs a) {
     vf.load(vt, rows, a.sv.s, d_v, tid);
     kt += (int64_t)kBC * a.sk.s; vt += (int64_t)kBC * a.sv.s; rows_left -= kBC;
   };
-  auto publish = [&]() { kf.store(Ks, tid); vf.store(Vs, tid); };
+  constexpr bool kTwoK = SM::K_STAGES == 2;
+  auto publish_k = [&](int stage) { kf.store(Ks + stage * (C::TILE_BYTES / 4), tid); };
+  auto publish_v = [&]() { vf.store(Vs, tid); };
 
   const float* bptr = nullptr;
   if (kBias)
@@ -293,15 +302,22 @@ __global__ __launch_bounds__(Cfg<D>::NT) void fwd_f32_kernel(const FwdArgs a) {
   const unsigned m_rng = m_none ? 0u : (unsigned)(m_hi - m_lo);
 
   fetch();
-  publish();
+  publish_k(0);
+  publish_v();
   __syncthreads();
   for (int j = br.lo; j <= br.hi; ++j) {
-    if (j < br.hi) fetch();
+    const int stage = kTwoK ? (j - br.lo) & 1 : 0;
+    if (!kTwoK && j < br.hi) fetch();
     // this wave's share of S^T = K Q^T
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    s = row_gemm<D>(Ks, c, hi, col0, qreg, s);
+    s = row_gemm<D>(Ks + stage * (C::TILE_BYTES / 4), c, hi, col0, qreg, s);
+    if (kTwoK) {
+      // behind the MFMAs: V of this tile goes to its stage, then the staging registers take the next tile
+      if (j > br.lo) publish_v();
+      if (j < br.hi) fetch();
+    }
     part_write(part, cw, lane, s);
     __syncthreads();
     s = part_sum(part, lane);
@@ -360,10 +376,16 @@ __global__ __launch_bounds__(Cfg<D>::NT) void fwd_f32_kernel(const FwdArgs a) {
     }
     // O^T += V^T P^T on this wave's columns
     col_gemm<D>(Vs, c, hi, col0, s, o);
-    __syncthreads();                 // the tile and the partial blocks have been read
-    if (j < br.hi) {
-      publish();
-      __syncthreads();
+    if (kTwoK) {
+      if (j < br.hi) publish_k(stage ^ 1);
+      __syncthreads();               // V and the partial blocks have been read, the next K is in place
+    } else {
+      __syncthreads();               // the tile and the partial blocks have been read
+      if (j < br.hi) {
+        publish_k(0);
+        publish_v();
+        __syncthreads();
+      }
     }
   }
 
